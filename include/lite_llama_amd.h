@@ -562,11 +562,22 @@ int ll_sample_top_p(int64_t* out, const void* logits, const float* temperature, 
  * ll_add_rmsnorm_shift: s = x_in + delta (delta may be NULL; else s is written to x_out), h = s / sqrt(mean(s^2) + eps) * w,
  * y = h + (h_prev - h) * shift (shift may be NULL: y = h), h_prev = h of the sequence's previous token (zeros at position
  * 0; from the state slot at the start of a run).  state = [2][state_half] floats, half seq_parity[i] is read and the other
- * half written (h of the run's last token, at slot * width).  x_out must differ from x_in when delta and shift are given. */
+ * half written (h of the run's last token, at slot * width).  x_out must differ from x_in when delta and shift are given.
+ * parts [n][num_parts][width] (or NULL): further rows of the update, s = x_in + (delta + (part_0 + part_1 + ..)).
+ * y is multiplied by out_scale (fp32, before the one rounding to dtype). */
 int ll_add_rmsnorm_shift(const float* x_in, const void* delta, float* x_out, const void* weight, const void* shift,
                          void* y, int64_t n, int64_t width, float eps, const int32_t* tok_seq,
                          const int32_t* seq_start, const int32_t* seq_first_pos, const int32_t* seq_slot,
-                         const int32_t* seq_parity, float* state, int64_t state_half, int dtype, void* stream);
+                         const int32_t* seq_parity, float* state, int64_t state_half, const void* parts, int64_t num_parts,
+                         float out_scale, int dtype, void* stream);
+/* x [n, width] (fp32) = embed[tokens[t]] * scale + pair[row]; row = (previous token * mul_prev + token * mul_cur) mod buckets,
+ * or `buckets` (the last row of pair [buckets + 1, width]) at position 0.  The previous token of a run's first token is read
+ * from prev_state [2][state_half] (half seq_parity, entry seq_slot); a run's last token is written to the other half.
+ * pair == NULL: no table, no state. */
+int ll_embed_pair(float* x, const int32_t* tokens, const void* embed, int64_t vocab, float scale, const void* pair,
+                  int64_t buckets, int64_t mul_prev, int64_t mul_cur, int64_t n, int64_t width, const int32_t* tok_seq,
+                  const int32_t* seq_start, const int32_t* seq_first_pos, const int32_t* seq_slot, const int32_t* seq_parity,
+                  int32_t* prev_state, int64_t state_half, int dtype, void* stream);
 /* xIELU with pq = (p, q): z > 0: softplus(p) z^2 + z / 2;  else (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2. */
 int ll_xielu(void* y, const void* z, const void* pq, int64_t n, int dtype, void* stream);
 /* out [n, 2 width] = [a + a_delta | b] cast to dtype (a_delta in dtype, or NULL);  x [n, width] (fp32) = y + bias (bias
@@ -594,12 +605,27 @@ int ll_qk_norm_cache(const void* qkv, int64_t ld, const void* q_w, const void* k
                      void* stream);
 /* Causal softmax attention of every token against positions 0 .. tok_pos[t] of its sequence (cache rows through
  * token_table[seq_req[tok_seq[t]]][pos]); score = (q . k) scale; sink [heads] or NULL adds exp(sink_h) to the denominator.
- * window > 0: only the last `window` positions (the token's own included) are seen.  k_stride / v_stride: elements between
- * cache rows (>= kv_heads dk / kv_heads dv; the value rows may be a column range of the key rows). */
+ * window > 0: only the last `window` positions (the token's own included) are seen, and besides them the sequence's first
+ * keep_first positions.  k_stride / v_stride: elements between cache rows (>= kv_heads dk / kv_heads dv; the value rows may
+ * be a column range of the key rows); out_stride: elements between output rows (>= heads dv). */
 int ll_ragged_attention(const void* q, const void* k_cache, const void* v_cache, const int32_t* token_table,
                         int64_t tt_stride, const int32_t* seq_req, const int32_t* tok_seq, const int32_t* tok_pos,
                         const void* sink, float scale, void* out, int64_t n, int64_t heads, int64_t kv_heads, int64_t dk,
-                        int64_t dv, int64_t k_stride, int64_t v_stride, int64_t window, int dtype, void* stream);
+                        int64_t dv, int64_t k_stride, int64_t v_stride, int64_t window, int64_t keep_first,
+                        int64_t out_stride, int dtype, void* stream);
+/* Rows [q (heads dk) | k (kv_heads dk) | v (kv_heads dv)] of stride ld, channel by channel in fp32: + bias [channels] (or NULL);
+ * y_t = sum_j conv_w[c][j] u_(t - taps + 1 + j) over the sequence's positions (zeros in front of position 0; taps == 0: none),
+ * the raw rows of a sequence's last taps - 1 positions carried in conv_state [2][state_half] (half seq_parity read, the other
+ * written; a slot is [taps - 1][channels], row d - 1 = position length - d); pairs (2i, 2i + 1), i < pairs, of every q / k head
+ * rotated by pos * freq[i] with cos / sin times amp; q / k heads divided by sqrt(mean + eps) when unit_norm; v = (1 - lam) v +
+ * lam v_src[select[t]] when v_src (rows of stride v_src_stride; lam = *v_lam) is given.  q -> q_out [n, heads, dk]; k, v ->
+ * cache rows select[t]. */
+int ll_conv_rope_cache(const void* qkv, int64_t ld, const void* bias, const void* conv_w, int64_t taps, void* conv_state,
+                       int64_t state_half, const float* freq, int64_t pairs, float amp, int unit_norm, float eps,
+                       const void* v_src, int64_t v_src_stride, const void* v_lam, const int32_t* tok_seq,
+                       const int32_t* tok_pos, const int32_t* select, const int32_t* seq_start, const int32_t* seq_first_pos,
+                       const int32_t* seq_slot, const int32_t* seq_parity, void* q_out, void* k_cache, void* v_cache,
+                       int64_t n, int64_t heads, int64_t kv_heads, int64_t dk, int64_t dv, int dtype, void* stream);
 /* MFMA form for 16-bit storage dtypes (dk, dv multiples of 8, <= 256).  decode == 0: prompt portions (16 consecutive tokens
  * of a run per wave; longest_run = most tokens a sequence brings).  decode != 0: every sequence brings one token (n == batch);
  * the query heads of a key/value head share a wave, the context is cut into partitions of ll_ragged_attention_partition()
@@ -612,7 +638,7 @@ int ll_ragged_attention_mfma(const void* q, const void* k_cache, const void* v_c
                              const int32_t* seq_first_pos, const void* sink, float scale, void* out, int64_t n,
                              int64_t batch, int64_t longest_run, int64_t longest_context, int decode, float* partials,
                              int64_t heads, int64_t kv_heads, int64_t dk, int64_t dv, int64_t k_stride, int64_t v_stride,
-                             int64_t window, int dtype, void* stream);
+                             int64_t window, int64_t keep_first, int64_t out_stride, int dtype, void* stream);
 
 /* ---- sublayers between two grouped norms with a gated residual branch (csrc/group_norm.hip) --------------------------------
  * ll_gated_group_norm: with y: s = (sum of `parts` rows y[t][p][:] + shared_scale[t] * shared[t][:]) * sigmoid(gate[t][:] +
@@ -623,10 +649,10 @@ int ll_gated_group_norm(const float* x_in, float* x_out, void* h_out, const void
                         const float* shared_scale, const void* gate, int64_t gate_ld, const void* gate_bias,
                         const void* post_w, const void* next_w, int64_t n, int64_t width, int64_t groups, float eps,
                         int dtype, void* stream);
-/* out [n, ff] = act(gate[t][j]) * up[t][j], gate / up rows of stride gate_ld / up_ld; kind 0: silu, 1: gelu (tanh form),
- * 2: sigmoid. */
-int ll_glu_act(void* out, const void* gate, int64_t gate_ld, const void* up, int64_t up_ld, int64_t n, int64_t ff, int kind,
-               int dtype, void* stream);
+/* out [n, ff] (rows of stride out_ld) = act(gate[t][j]) * up[t][j], gate / up rows of stride gate_ld / up_ld; kind 0: silu,
+ * 1: gelu (tanh form), 2: sigmoid, 3: clamped -- g = min(gate, p0), u = clamp(up, -p0, p0), g sigmoid(p1 g) (u + 1). */
+int ll_glu_act(void* out, int64_t out_ld, const void* gate, int64_t gate_ld, const void* up, int64_t up_ld, int64_t n,
+               int64_t ff, int kind, float p0, float p1, int dtype, void* stream);
 /* x <- cap * tanh(x / cap), in place. */
 int ll_softcap(void* x, int64_t n, float cap, int dtype, void* stream);
 /* minGRU: rows [z | x | g] (three pointers, one stride ld): z = sigmoid(z_raw + z_bias), u = x_raw + x_bias, candidate u + 1/2
@@ -658,13 +684,14 @@ int ll_rotate_pairs(const void* q, int64_t q_tok_stride, int64_t q_head_stride, 
  * ll_group_router: scores = sigmoid(W_router h) in fp32; experts in group_count equal groups of neighbours, group score = sum
  * of its two best, the best group_keep groups stay eligible; ids [n, top] / weights [n, top] (fp32) = the top eligible experts
  * by score and score / (sum + 1e-20) * route_scale.  w_extra [width] (or NULL): extra_scale[t] = sigmoid(w_extra . h).
- * logits: fp32 scratch [n][experts + (w_extra ? 1 : 0)].
+ * logits: fp32 scratch [n][experts + (w_extra ? 1 : 0)].  scoring 1: no sigmoid and no groups -- the `top` largest logits
+ * are chosen and their weights are the softmax over the chosen logits alone (times route_scale).
  * ll_moe_sort: slots sorted by expert in blocks of `block` = ll_moe_rows_block(...) rows, 32 or 128 (counts: int32 scratch
  * [experts]; sorted [num_slots + experts (block - 1)], block_expert [ceil(that / block)], num_post [1]).
  * ll_moe_rows_gemm: glu != 0: w [experts][2 N][K] (gate rows, then up rows), out[slot] = silu(a Wg^T) * (a Wu^T) with
  * a = row slot / a_div; glu == 0: w [experts][N][K], out[slot] = (a W^T) * slot_weight[slot]. */
 int ll_group_router(const void* h, int64_t h_ld, const void* w_router, const void* w_extra, int64_t n, int64_t width,
-                    int64_t experts, int64_t top, int64_t group_count, int64_t group_keep, float route_scale,
+                    int64_t experts, int64_t top, int64_t group_count, int64_t group_keep, float route_scale, int scoring,
                     int32_t* ids, float* weights, float* extra_scale, float* logits, int dtype, void* stream);
 int64_t ll_moe_rows_block(int64_t num_slots, int64_t experts, int64_t width, int64_t ff, int dtype);
 int ll_moe_sort(const int32_t* ids, int64_t num_slots, int64_t experts, int64_t block, int32_t* counts, int32_t* sorted,

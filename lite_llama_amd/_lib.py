@@ -110,25 +110,27 @@ SIGNATURES = {
     "ll_repetition_penalty": [P, P, P, P, P, F, L, L, L, L, L, L, L, I, I, P],
     "ll_sample_top_p": [P, P, P, P, P, P, L, L, L, I, P],
     "ll_argmax_split": [P, P, L, L, L, I, P, I, P],
-    "ll_add_rmsnorm_shift": [P, P, P, P, P, P, L, L, F, P, P, P, P, P, P, L, I, P],
+    "ll_add_rmsnorm_shift": [P, P, P, P, P, P, L, L, F, P, P, P, P, P, P, L, P, L, F, I, P],
+    "ll_embed_pair": [P, P, P, L, F, P, L, L, L, L, L, P, P, P, P, P, P, L, I, P],
     "ll_xielu": [P, P, P, L, I, P],
     "ll_cast_pair": [P, P, P, P, L, L, I, P],
     "ll_residual_set": [P, P, P, L, L, I, P],
     "ll_gated_linear_scan_supported": [L, L],
     "ll_gated_linear_scan": [P, P, P, L, P, P, P, F, P, L, L, L, L, P, P, P, P, L, L, P, I, P],
     "ll_qk_norm_cache": [P, L, P, P, F, F, L, P, P, P, P, P, L, L, L, L, L, I, P],
-    "ll_ragged_attention": [P, P, P, P, L, P, P, P, P, F, P, L, L, L, L, L, L, L, L, I, P],
+    "ll_ragged_attention": [P, P, P, P, L, P, P, P, P, F, P, L, L, L, L, L, L, L, L, L, L, I, P],
+    "ll_conv_rope_cache": [P, L, P, P, L, P, L, P, L, F, I, F, P, L, P, P, P, P, P, P, P, P, P, P, P, L, L, L, L, L, I, P],
     "ll_ragged_attention_mfma_supported": [L, L, I],
     "ll_ragged_attention_partition": [],
-    "ll_ragged_attention_mfma": [P, P, P, P, L, P, P, P, P, F, P, L, L, L, L, I, P, L, L, L, L, L, L, L, I, P],
+    "ll_ragged_attention_mfma": [P, P, P, P, L, P, P, P, P, F, P, L, L, L, L, I, P, L, L, L, L, L, L, L, L, L, I, P],
     "ll_gated_group_norm": [P, P, P, P, L, P, P, P, L, P, P, P, L, L, L, F, I, P],
-    "ll_glu_act": [P, P, L, P, L, L, L, I, I, P],
+    "ll_glu_act": [P, L, P, L, P, L, L, L, I, F, F, I, P],
     "ll_softcap": [P, L, F, I, P],
     "ll_mingru_scan_scratch_floats": [L, L, L],
     "ll_mingru_scan": [P, P, P, L, P, P, P, L, L, P, P, P, P, L, P, I, P],
     "ll_latent_kv_prep": [P, L, L, L, L, P, F, P, L, F, P, P, P, L, L, L, P, P, L, I, P],
     "ll_rotate_pairs": [P, L, L, L, L, P, L, F, P, P, L, L, L, L, I, P],
-    "ll_group_router": [P, L, P, P, L, L, L, L, L, L, F, P, P, P, P, I, P],
+    "ll_group_router": [P, L, P, P, L, L, L, L, L, L, F, I, P, P, P, P, I, P],
     "ll_moe_rows_block": [L, L, L, L, I],
     "ll_moe_sort": [P, L, L, L, P, P, P, P, P],
     "ll_moe_rows_gemm": [P, L, L, P, L, L, L, I, P, P, L, P, P, P, L, L, L, I, P],

@@ -9,7 +9,9 @@
 //                         sum of several rows -- the experts a token chose -- plus a scaled shared row) times the sigmoid of its
 //                         gate logits, grouped norm with the post weight, residual add in fp32, then the grouped norm that feeds
 //                         the next sublayer (or the output head).  Without a pending result it is the plain grouped norm.
-//   ll_glu_act            act(gate) * up, gate and up two row-strided column ranges (act: silu, the tanh form of gelu, sigmoid)
+//   ll_glu_act            act(gate) * up, gate and up two row-strided column ranges (act: silu, the tanh form of gelu, sigmoid),
+//                         or the clamped form g sigmoid(a g) (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit);
+//                         the result may be a column range of wider rows
 //
 // Storage dtype DT = LL_F16 / LL_BF16 / LL_F32 for activations and weights; sums, norms, gates and the residual are fp32.
 #include "common.h"
@@ -270,25 +272,19 @@ template <int DT>
 __device__ __forceinline__ float glu_value(float g, float u, int kind);
 
 // out[t][j] = act(gate[t][j]) * up[t][j]; gate and up rows have their own strides (two column ranges of one projection, or two
-// tensors).  kind 0: silu, 1: gelu (tanh form), 2: sigmoid
+// tensors).  kind 0: silu, 1: gelu (tanh form), 2: sigmoid, 3: clamped (p0 = limit, p1 = slope inside the sigmoid)
 template <int DT>
-__global__ __launch_bounds__(256) void glu_act_kernel(void* __restrict__ out, const void* __restrict__ gate, int64_t gate_ld,
-                                                      const void* __restrict__ up, int64_t up_ld, int64_t n, int ff, int kind) {
-  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= n * ff) return;
-  const int64_t t = idx / ff;
-  const int j = (int)(idx - t * ff);
-  stv<DT>(out, idx, glu_value<DT>(ldv<DT>(gate, t * gate_ld + j), ldv<DT>(up, t * up_ld + j), kind));
-}
-
-template <int DT>
-__device__ __forceinline__ float glu_value(float g, float u, int kind) {
+__device__ __forceinline__ float glu_value(float g, float u, int kind, float p0, float p1) {
   constexpr bool EXACT = DT == LL_F32;
   float a;
   if (kind == 0) {
     a = g * sigmoid_f<EXACT>(g);
   } else if (kind == 2) {
     a = sigmoid_f<EXACT>(g);
+  } else if (kind == 3) {
+    g = fminf(g, p0);
+    u = fminf(fmaxf(u, -p0), p0) + 1.0f;
+    a = g * sigmoid_f<EXACT>(p1 * g);
   } else {
     const float inner = 0.7978845608028654f * (g + 0.044715f * g * g * g);
     const float th = EXACT ? tanhf(inner) : 2.0f * ll_sigmoidf(2.0f * inner) - 1.0f;
@@ -297,10 +293,22 @@ __device__ __forceinline__ float glu_value(float g, float u, int kind) {
   return a * u;
 }
 
+template <int DT>
+__global__ __launch_bounds__(256) void glu_act_kernel(void* __restrict__ out, int64_t out_ld, const void* __restrict__ gate,
+                                                      int64_t gate_ld, const void* __restrict__ up, int64_t up_ld, int64_t n, int ff,
+                                                      int kind, float p0, float p1) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= n * ff) return;
+  const int64_t t = idx / ff;
+  const int j = (int)(idx - t * ff);
+  stv<DT>(out, t * out_ld + j, glu_value<DT>(ldv<DT>(gate, t * gate_ld + j), ldv<DT>(up, t * up_ld + j), kind, p0, p1));
+}
+
 // 16-byte form: a thread owns one piece (8 sixteen-bit / 4 fp32 values) of a row; same values as the plain form
 template <int DT>
-__global__ __launch_bounds__(256) void glu_act_vec_kernel(void* __restrict__ out, const void* __restrict__ gate, int64_t gate_ld,
-                                                          const void* __restrict__ up, int64_t up_ld, int64_t n, int ff, int kind) {
+__global__ __launch_bounds__(256) void glu_act_vec_kernel(void* __restrict__ out, int64_t out_ld, const void* __restrict__ gate,
+                                                          int64_t gate_ld, const void* __restrict__ up, int64_t up_ld, int64_t n,
+                                                          int ff, int kind, float p0, float p1) {
   constexpr int VEC = DT == LL_F32 ? 4 : 8;
   const int pieces = ff / VEC;
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -312,15 +320,15 @@ __global__ __launch_bounds__(256) void glu_act_vec_kernel(void* __restrict__ out
     const f32x4 u = *reinterpret_cast<const f32x4*>((const float*)up + t * up_ld + j);
     f32x4 o;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) o[i] = glu_value<DT>(g[i], u[i], kind);
-    *reinterpret_cast<f32x4*>((float*)out + t * ff + j) = o;
+    for (int i = 0; i < 4; ++i) o[i] = glu_value<DT>(g[i], u[i], kind, p0, p1);
+    *reinterpret_cast<f32x4*>((float*)out + t * out_ld + j) = o;
   } else {
     const U16x8 g = *reinterpret_cast<const U16x8*>((const uint16_t*)gate + t * gate_ld + j);
     const U16x8 u = *reinterpret_cast<const U16x8*>((const uint16_t*)up + t * up_ld + j);
     U16x8 o;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) o.v[i] = from_f32<DT>(glu_value<DT>(to_f32<DT>(g.v[i]), to_f32<DT>(u.v[i]), kind));
-    *reinterpret_cast<U16x8*>((uint16_t*)out + t * ff + j) = o;
+    for (int i = 0; i < 8; ++i) o.v[i] = from_f32<DT>(glu_value<DT>(to_f32<DT>(g.v[i]), to_f32<DT>(u.v[i]), kind, p0, p1));
+    *reinterpret_cast<U16x8*>((uint16_t*)out + t * out_ld + j) = o;
   }
 }
 
@@ -378,23 +386,23 @@ extern "C" int ll_gated_group_norm(const float* x_in, float* x_out, void* h_out,
   return LL_LAUNCH_CHECK();
 }
 
-extern "C" int ll_glu_act(void* out, const void* gate, int64_t gate_ld, const void* up, int64_t up_ld, int64_t n, int64_t ff,
-                          int kind, int dtype, void* stream) {
+extern "C" int ll_glu_act(void* out, int64_t out_ld, const void* gate, int64_t gate_ld, const void* up, int64_t up_ld, int64_t n,
+                          int64_t ff, int kind, float p0, float p1, int dtype, void* stream) {
   if (dtype != LL_F16 && dtype != LL_BF16 && dtype != LL_F32) return LL_ERR_DTYPE;
-  if (n < 0 || ff < 1 || gate_ld < ff || up_ld < ff || ff > (1 << 24) || kind < 0 || kind > 2) return LL_ERR_SHAPE;
+  if (n < 0 || ff < 1 || out_ld < ff || gate_ld < ff || up_ld < ff || ff > (1 << 24) || kind < 0 || kind > 3) return LL_ERR_SHAPE;
   if (n == 0) return LL_OK;
   if (!out || !gate || !up) return LL_ERR_ARG;
   hipStream_t st = (hipStream_t)stream;
   const int vec = dtype == LL_F32 ? 4 : 8;
-  if (ff % vec == 0 && gate_ld % vec == 0 && up_ld % vec == 0 && ll_aligned16(out) && ll_aligned16(gate) && ll_aligned16(up)) {
+  if (ff % vec == 0 && out_ld % vec == 0 && gate_ld % vec == 0 && up_ld % vec == 0 && ll_aligned16(out) && ll_aligned16(gate) && ll_aligned16(up)) {
     const dim3 grid((unsigned)((n * (ff / vec) + 255) / 256));
-#define CALL(DT) glu_act_vec_kernel<DT><<<grid, 256, 0, st>>>(out, gate, gate_ld, up, up_ld, n, (int)ff, kind)
+#define CALL(DT) glu_act_vec_kernel<DT><<<grid, 256, 0, st>>>(out, out_ld, gate, gate_ld, up, up_ld, n, (int)ff, kind, p0, p1)
     LL_BY_DTYPE(dtype, CALL);
 #undef CALL
     return LL_LAUNCH_CHECK();
   }
   const dim3 grid((unsigned)((n * ff + 255) / 256));
-#define CALL(DT) glu_act_kernel<DT><<<grid, 256, 0, st>>>(out, gate, gate_ld, up, up_ld, n, (int)ff, kind)
+#define CALL(DT) glu_act_kernel<DT><<<grid, 256, 0, st>>>(out, out_ld, gate, gate_ld, up, up_ld, n, (int)ff, kind, p0, p1)
   LL_BY_DTYPE(dtype, CALL);
 #undef CALL
   return LL_LAUNCH_CHECK();

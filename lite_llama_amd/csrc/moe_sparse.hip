@@ -102,8 +102,9 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const void* __restri
 }
 
 // router, second launch: one 64-thread workgroup per token over its logits.  LDS: scores [E], group score [G], group kept
-// [G], chosen scores [top]
-template <int DUMMY>
+// [G], chosen scores [top].  SCORING 0: sigmoid scores, weights = chosen / sum; 1: the logits themselves rank the experts (no
+// groups) and the weights are the softmax over the chosen logits alone
+template <int SCORING>
 __global__ __launch_bounds__(64) void group_select_kernel(const float* __restrict__ logits, int rows, int experts, int top,
                                                           int group_count, int group_keep, float route_scale,
                                                           int32_t* __restrict__ ids, float* __restrict__ weights,
@@ -116,9 +117,9 @@ __global__ __launch_bounds__(64) void group_select_kernel(const float* __restric
   const int64_t t = blockIdx.x;
   const int lane = threadIdx.x;
   for (int e = lane; e < rows; e += 64) {
-    const float s = sigmoid_exact(logits[t * rows + e]);
-    if (e < experts) score[e] = s;
-    else extra_scale[t] = s;
+    const float z = logits[t * rows + e];
+    if (e < experts) score[e] = SCORING == 1 ? z : sigmoid_exact(z);
+    else extra_scale[t] = sigmoid_exact(z);
   }
   __syncthreads();
   const int per = experts / group_count;
@@ -157,8 +158,13 @@ __global__ __launch_bounds__(64) void group_select_kernel(const float* __restric
   }
   __syncthreads();
   float sum = 0.f;
-  for (int k = 0; k < top; ++k) sum += chosen[k];
-  for (int k = lane; k < top; k += 64) weights[t * top + k] = chosen[k] / (sum + 1e-20f) * route_scale;
+  if constexpr (SCORING == 1) {   // chosen[0] is the largest: exp(z - z_max) summed in slot order by every lane
+    for (int k = 0; k < top; ++k) sum += expf(chosen[k] - chosen[0]);
+    for (int k = lane; k < top; k += 64) weights[t * top + k] = expf(chosen[k] - chosen[0]) / sum * route_scale;
+  } else {
+    for (int k = 0; k < top; ++k) sum += chosen[k];
+    for (int k = lane; k < top; k += 64) weights[t * top + k] = chosen[k] / (sum + 1e-20f) * route_scale;
+  }
 }
 
 // ------------------------------------------------------------------------------------------------------------------------
@@ -475,11 +481,12 @@ __global__ __launch_bounds__(256) void moe_rows_gemm_tiled_kernel(const uint16_t
 
 // logits: fp32 scratch [n][experts + (w_extra ? 1 : 0)]
 extern "C" int ll_group_router(const void* h, int64_t h_ld, const void* w_router, const void* w_extra, int64_t n, int64_t width,
-                               int64_t experts, int64_t top, int64_t group_count, int64_t group_keep, float route_scale,
+                               int64_t experts, int64_t top, int64_t group_count, int64_t group_keep, float route_scale, int scoring,
                                int32_t* ids, float* weights, float* extra_scale, float* logits, int dtype, void* stream) {
   if (dtype != LL_F16 && dtype != LL_BF16 && dtype != LL_F32) return LL_ERR_DTYPE;
   if (n < 0 || width < 1 || h_ld < width || experts < 1 || experts > 4096 || top < 1 || top > experts || top > 64 || group_count < 1 ||
-      experts % group_count || group_keep < 1 || group_keep > group_count || group_keep * (experts / group_count) < top)
+      experts % group_count || group_keep < 1 || group_keep > group_count || group_keep * (experts / group_count) < top ||
+      scoring < 0 || scoring > 1 || (scoring == 1 && group_count != 1))
     return LL_ERR_SHAPE;
   if (n == 0) return LL_OK;
   if (!h || !w_router || !ids || !weights || !logits || (w_extra && !extra_scale)) return LL_ERR_ARG;
@@ -507,8 +514,12 @@ extern "C" int ll_group_router(const void* h, int64_t h_ld, const void* w_router
 #undef LL_RL
 #undef LL_RL_ARGS
   const size_t lds = sizeof(float) * (size_t)(experts + 2 * group_count + top);
-  group_select_kernel<0><<<dim3((unsigned)n), 64, lds, st>>>(logits, rows, (int)experts, (int)top, (int)group_count, (int)group_keep,
-                                                             route_scale, ids, weights, extra_scale);
+  if (scoring == 1)
+    group_select_kernel<1><<<dim3((unsigned)n), 64, lds, st>>>(logits, rows, (int)experts, (int)top, (int)group_count, (int)group_keep,
+                                                               route_scale, ids, weights, extra_scale);
+  else
+    group_select_kernel<0><<<dim3((unsigned)n), 64, lds, st>>>(logits, rows, (int)experts, (int)top, (int)group_count, (int)group_keep,
+                                                               route_scale, ids, weights, extra_scale);
   return LL_LAUNCH_CHECK();
 }
 

@@ -4,8 +4,13 @@
 //
 //   ll_qk_norm_cache     fused projection rows [q | k | v] -> normed, temperature-scaled queries; normed keys and raw values
 //                        written to the cache rows of their tokens
+//   ll_conv_rope_cache   fused projection rows [q | k | v] -> bias, a short causal convolution over time per channel (the last
+//                        taps - 1 projected rows of a sequence are carried in a state slot), rotation of entry pairs of q / k
+//                        heads, unit RMS norm of q / k heads, values blended with the values another layer cached for the same
+//                        token; queries out, keys and values into the cache rows of their tokens
 //   ll_ragged_attention  every token of the step against keys 0 .. its own position of its sequence, read through the
-//                        per-token row table; scores, softmax and the running output in fp32
+//                        per-token row table; scores, softmax and the running output in fp32; optionally only the last
+//                        `window` keys plus the sequence's first `keep_first`
 //
 // The sink is a virtual key with score sink_h (not scaled) and a zero value: the running softmax simply STARTS at
 // (max = sink, sum = 1, output = 0).  A token's result depends only on its own position and on the cache rows of its
@@ -64,6 +69,117 @@ __global__ __launch_bounds__(256) void qk_norm_cache_kernel(
     if (wt) r *= ldv<DT>(wt, c);
     if (is_q) stv<DT>(q_out, (t * heads + item) * dk + c, r * temp);
     else stv<DT>(k_cache, (row * kv_heads + (item - heads)) * dk + c, r);
+  }
+}
+
+// One wave per (token, item): items 0 .. H - 1 = query heads, H .. H + G - 1 = key heads, then G value heads.  Lane l owns the
+// entry pairs l, l + 64, .. of its head (NP of them).  Per channel, in fp32:
+//   u_p   = projected row of position p (+ bias): this step's rows, or -- in front of the run -- the sequence's state slot, which
+//           holds the RAW projected rows of its last taps - 1 positions (row d - 1 = position length - d); zeros in front of
+//           position 0
+//   y     = sum_j w[c][j] u_(pos - taps + 1 + j)                       (taps == 0: y = u)
+//   q, k  : pairs (2i, 2i + 1), i < pairs, rotated by pos * freq[i] with cos / sin times amp; then the head divided by
+//           sqrt(mean(y^2) + eps) when unit_norm
+//   v     : (1 - lam) y + lam v_src[select[t]] when a source cache is given
+// The wave of a run's LAST token also writes its item's channels of the state slot for the next step (other half of the pair).
+template <int DT, int NP>
+__global__ __launch_bounds__(256) void conv_rope_cache_kernel(
+    const void* __restrict__ qkv, int64_t ld, const void* __restrict__ bias, const void* __restrict__ conv_w, int taps,
+    void* __restrict__ conv_state, int64_t state_half, const float* __restrict__ freq, int pairs, float amp, int unit_norm,
+    float eps, const void* __restrict__ v_src, int64_t v_src_stride, const void* __restrict__ v_lam,
+    const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ select,
+    const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_first_pos, const int32_t* __restrict__ seq_slot,
+    const int32_t* __restrict__ seq_parity, void* __restrict__ q_out, void* __restrict__ k_cache, void* __restrict__ v_cache,
+    int64_t n, int heads, int kv_heads, int dk, int dv) {
+  const int items = heads + 2 * kv_heads;
+  const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (w >= n * items) return;
+  const int lane = threadIdx.x & 63;
+  const int64_t t = w / items;
+  const int item = (int)(w - t * items);
+  const bool is_q = item < heads, is_v = item >= heads + kv_heads;
+  const int width = is_v ? dv : dk;
+  const int64_t col0 = is_v ? (int64_t)(heads + kv_heads) * dk + (int64_t)(item - heads - kv_heads) * dv : (int64_t)item * dk;
+  const int64_t channels = (int64_t)(heads + kv_heads) * dk + (int64_t)kv_heads * dv;
+  const int b = tok_seq[t];
+  const int pos = tok_pos[t], first = seq_first_pos[b];
+  const int in_run = pos - first;                       // tokens of the run in front of this one
+  const int back = taps > 1 ? taps - 1 : 0;
+  const uint8_t* old_state = nullptr;
+  if (back) old_state = (const uint8_t*)conv_state + ((int64_t)seq_parity[b] * state_half + (int64_t)seq_slot[b] * back * channels) *
+                                                         (DT == LL_F32 ? 4 : 2);
+  // projected value (+ bias) of channel c at `d` positions in front of this token (d = 0: its own); 0 in front of position 0
+  auto u_at = [&](int64_t c, int d) -> float {
+    if (d > pos) return 0.f;
+    float v;
+    if (d <= in_run) v = ldv<DT>(qkv, (t - d) * ld + c);
+    else v = ldv<DT>(old_state, (int64_t)(d - in_run - 1) * channels + c);
+    return bias ? v + ldv<DT>(bias, c) : v;
+  };
+  auto conv_at = [&](int64_t c) -> float {
+    if (taps <= 0) return u_at(c, 0);
+    float y = 0.f;
+    for (int j = 0; j < taps; ++j) y += ldv<DT>(conv_w, c * taps + j) * u_at(c, taps - 1 - j);
+    return y;
+  };
+  float a[NP], bb[NP];
+  float ss = 0.f;
+  const float fpos = (float)pos;
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    const int pi = lane + 64 * i;
+    a[i] = bb[i] = 0.f;
+    if (2 * pi < width) {
+      a[i] = conv_at(col0 + 2 * pi);
+      if (2 * pi + 1 < width) bb[i] = conv_at(col0 + 2 * pi + 1);
+      if (!is_v && pi < pairs) {
+        const float ang = fpos * freq[pi];
+        const float cs = cosf(ang) * amp, sn = sinf(ang) * amp;
+        const float x0 = a[i], x1 = bb[i];
+        a[i] = x0 * cs - x1 * sn;
+        bb[i] = x1 * cs + x0 * sn;
+      }
+      ss += a[i] * a[i];
+      ss += bb[i] * bb[i];
+    }
+  }
+  float mul = 1.0f, lam = 0.f;
+  if (!is_v && unit_norm) {
+    ss = wave_sum(ss);
+    mul = 1.0f / sqrtf(ss / (float)dk + eps);
+  }
+  const int64_t crow = select[t];
+  const bool blend = is_v && v_src != nullptr;
+  if (blend) lam = ldv<DT>(v_lam, 0);
+  const int64_t dst = is_q ? (t * heads + item) * dk
+                           : is_v ? (crow * kv_heads + (item - heads - kv_heads)) * dv : (crow * kv_heads + (item - heads)) * dk;
+  void* dstp = is_q ? q_out : is_v ? v_cache : k_cache;
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    const int pi = lane + 64 * i;
+    if (2 * pi < width) {
+      float y0 = a[i] * mul, y1 = bb[i] * mul;
+      if (blend) {
+        const int64_t src = crow * v_src_stride + (int64_t)(item - heads - kv_heads) * dv + 2 * pi;
+        y0 = (1.0f - lam) * y0 + lam * ldv<DT>(v_src, src);
+        if (2 * pi + 1 < width) y1 = (1.0f - lam) * y1 + lam * ldv<DT>(v_src, src + 1);
+      }
+      stv<DT>(dstp, dst + 2 * pi, y0);
+      if (2 * pi + 1 < width) stv<DT>(dstp, dst + 2 * pi + 1, y1);
+    }
+  }
+  // the run's last token leaves the raw projected rows of the sequence's last taps - 1 positions
+  if (back && t == seq_start[b + 1] - 1) {
+    uint8_t* new_state = (uint8_t*)conv_state + ((int64_t)(1 - seq_parity[b]) * state_half + (int64_t)seq_slot[b] * back * channels) *
+                                                    (DT == LL_F32 ? 4 : 2);
+    for (int d = 1; d <= back; ++d) {                   // state row d - 1 = the position d - 1 in front of this token
+      for (int c = lane; c < width; c += 64) {
+        float v = 0.f;
+        if (d - 1 <= in_run) v = ldv<DT>(qkv, (t - (d - 1)) * ld + col0 + c);
+        else if (d - 1 <= pos) v = ldv<DT>(old_state, (int64_t)(d - 1 - in_run - 1) * channels + col0 + c);
+        stv<DT>(new_state, (int64_t)(d - 1) * channels + col0 + c, v);
+      }
+    }
   }
 }
 
@@ -184,7 +300,8 @@ __global__ __launch_bounds__(256) void ragged_attention_kernel(
     const void* __restrict__ q, const void* __restrict__ k_cache, const void* __restrict__ v_cache,
     const int32_t* __restrict__ token_table, int64_t tt_stride, const int32_t* __restrict__ seq_req,
     const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos, const void* __restrict__ sink, float scale,
-    void* __restrict__ out, int64_t n, int heads, int kv_heads, int dk, int dv, int64_t k_stride, int64_t v_stride, int window) {
+    void* __restrict__ out, int64_t n, int heads, int kv_heads, int dk, int dv, int64_t k_stride, int64_t v_stride, int window,
+    int keep_first, int64_t out_stride) {
   extern __shared__ float lds[];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   float* sq = lds + wave * (dk + 128);  // [dk] query
@@ -210,25 +327,28 @@ __global__ __launch_bounds__(256) void ragged_attention_kernel(
 #pragma unroll
   for (int i = 0; i < VPL; ++i) acc[i] = 0.f;
   __builtin_amdgcn_wave_barrier();
-  for (int base = first_key; base <= pos; base += 64) {
+  // keys in position order: the sequence's first `keep_first` keys that lie in front of the window, then the window
+  const int kept = keep_first < first_key ? keep_first : first_key;
+  for (int base = kept > 0 ? 0 : first_key; base <= pos; base = (base < first_key && base + 64 >= kept) ? first_key : base + 64) {
+    const int lim = base < first_key ? kept - 1 : pos;   // last key of this stretch
     const int j = base + lane;
     float s = -INFINITY;
     int row = 0;
-    if (j <= pos) {
+    if (j <= lim) {
       row = table[j];
       const int64_t kb = (int64_t)row * k_stride + (int64_t)g * dk;
       s = dot_row<DT>(sq, k_cache, kb, dk, vec) * scale;
     }
     const float tile_max = wave_max(s);
     const float m_new = fmaxf(m, tile_max);
-    const float p = j <= pos ? expf(s - m_new) : 0.f;
+    const float p = j <= lim ? expf(s - m_new) : 0.f;
     const float corr = m == -INFINITY ? 0.f : expf(m - m_new);
     l = l * corr + wave_sum(p);
     m = m_new;
     sp[lane] = p;
     sr[lane] = row;
     __builtin_amdgcn_wave_barrier();
-    const int cnt = pos - base + 1 < 64 ? pos - base + 1 : 64;
+    const int cnt = lim - base + 1 < 64 ? lim - base + 1 : 64;
 #pragma unroll
     for (int i = 0; i < VPL; ++i) {
       const int c = lane + 64 * i;
@@ -244,7 +364,7 @@ __global__ __launch_bounds__(256) void ragged_attention_kernel(
 #pragma unroll
   for (int i = 0; i < VPL; ++i) {
     const int c = lane + 64 * i;
-    if (c < dv) stv<DT>(out, (t * heads + h) * dv + c, acc[i] * inv);
+    if (c < dv) stv<DT>(out, t * out_stride + (int64_t)h * dv + c, acc[i] * inv);
   }
 }
 
@@ -283,13 +403,49 @@ extern "C" int ll_qk_norm_cache(const void* qkv, int64_t ld, const void* q_w, co
   return LL_LAUNCH_CHECK();
 }
 
+extern "C" int ll_conv_rope_cache(const void* qkv, int64_t ld, const void* bias, const void* conv_w, int64_t taps, void* conv_state,
+                                  int64_t state_half, const float* freq, int64_t pairs, float amp, int unit_norm, float eps,
+                                  const void* v_src, int64_t v_src_stride, const void* v_lam, const int32_t* tok_seq,
+                                  const int32_t* tok_pos, const int32_t* select, const int32_t* seq_start,
+                                  const int32_t* seq_first_pos, const int32_t* seq_slot, const int32_t* seq_parity, void* q_out,
+                                  void* k_cache, void* v_cache, int64_t n, int64_t heads, int64_t kv_heads, int64_t dk, int64_t dv,
+                                  int dtype, void* stream) {
+  if (dtype != LL_F16 && dtype != LL_BF16 && dtype != LL_F32) return LL_ERR_DTYPE;
+  if (n < 0 || heads < 1 || kv_heads < 1 || heads % kv_heads || dk < 1 || dk > 1024 || dv < 1 || dv > 1024 || taps < 0 || taps > 64 ||
+      pairs < 0 || 2 * pairs > dk || ld < (heads + kv_heads) * dk + kv_heads * dv || (v_src && v_src_stride < kv_heads * dv))
+    return LL_ERR_SHAPE;
+  if (n == 0) return LL_OK;
+  if (!qkv || !tok_seq || !tok_pos || !select || !seq_start || !seq_first_pos || !seq_slot || !seq_parity || !q_out || !k_cache ||
+      !v_cache || (taps > 0 && !conv_w) || (taps > 1 && !conv_state) || (pairs > 0 && !freq) || (v_src && !v_lam))
+    return LL_ERR_ARG;
+  const int64_t waves = n * (heads + 2 * kv_heads);
+  const dim3 grid((unsigned)((waves + 3) / 4));
+  const int64_t widest = dk > dv ? dk : dv;
+  hipStream_t st = (hipStream_t)stream;
+#define LL_CR_ARGS                                                                                                              \
+  qkv, ld, bias, conv_w, (int)taps, conv_state, state_half, freq, (int)pairs, amp, unit_norm, eps, v_src, v_src_stride, v_lam, tok_seq, \
+      tok_pos, select, seq_start, seq_first_pos, seq_slot, seq_parity, q_out, k_cache, v_cache, n, (int)heads, (int)kv_heads, (int)dk, \
+      (int)dv
+#define CALL(DT)                                                                               \
+  if (widest <= 128) conv_rope_cache_kernel<DT, 1><<<grid, 256, 0, st>>>(LL_CR_ARGS);          \
+  else if (widest <= 256) conv_rope_cache_kernel<DT, 2><<<grid, 256, 0, st>>>(LL_CR_ARGS);     \
+  else if (widest <= 512) conv_rope_cache_kernel<DT, 4><<<grid, 256, 0, st>>>(LL_CR_ARGS);     \
+  else conv_rope_cache_kernel<DT, 8><<<grid, 256, 0, st>>>(LL_CR_ARGS)
+  LL_BY_DTYPE(dtype, CALL);
+#undef CALL
+#undef LL_CR_ARGS
+  return LL_LAUNCH_CHECK();
+}
+
 extern "C" int ll_ragged_attention(const void* q, const void* k_cache, const void* v_cache, const int32_t* token_table,
                                    int64_t tt_stride, const int32_t* seq_req, const int32_t* tok_seq, const int32_t* tok_pos,
                                    const void* sink, float scale, void* out, int64_t n, int64_t heads, int64_t kv_heads, int64_t dk,
-                                   int64_t dv, int64_t k_stride, int64_t v_stride, int64_t window, int dtype, void* stream) {
+                                   int64_t dv, int64_t k_stride, int64_t v_stride, int64_t window, int64_t keep_first,
+                                   int64_t out_stride, int dtype, void* stream) {
   if (dtype != LL_F16 && dtype != LL_BF16 && dtype != LL_F32) return LL_ERR_DTYPE;
   if (n < 0 || heads < 1 || kv_heads < 1 || heads % kv_heads || dk < 1 || dk > 1024 || dv < 1 || dv > 1024 || window < 0 ||
-      window > 0x7fffffff || k_stride < kv_heads * dk || v_stride < kv_heads * dv)
+      window > 0x7fffffff || keep_first < 0 || keep_first > 0x7fffffff || k_stride < kv_heads * dk || v_stride < kv_heads * dv ||
+      out_stride < heads * dv)
     return LL_ERR_SHAPE;
   if (n == 0) return LL_OK;
   if (!q || !k_cache || !v_cache || !token_table || !seq_req || !tok_seq || !tok_pos || !out) return LL_ERR_ARG;
@@ -301,7 +457,7 @@ extern "C" int ll_ragged_attention(const void* q, const void* k_cache, const voi
 #define CALL_V(DT, V)                                                                                                        \
   ragged_attention_kernel<DT, V><<<grid, 256, lds, st>>>(q, k_cache, v_cache, token_table, tt_stride, seq_req, tok_seq, tok_pos, \
                                                          sink, scale, out, n, (int)heads, (int)kv_heads, (int)dk, (int)dv, k_stride, \
-                                                         v_stride, (int)window)
+                                                         v_stride, (int)window, (int)keep_first, out_stride)
 #define CALL(DT)                     \
   if (vpl == 1) CALL_V(DT, 1);       \
   else if (vpl == 2) CALL_V(DT, 2);  \

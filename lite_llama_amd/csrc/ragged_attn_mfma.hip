@@ -49,7 +49,7 @@ __global__ __launch_bounds__(64) void ragged_attention_mfma_decode_kernel(
     const int32_t* __restrict__ token_table, int64_t tt_stride, const int32_t* __restrict__ seq_req,
     const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_first_pos, const uint16_t* __restrict__ sink,
     float scale_log2, uint16_t* __restrict__ out, float* __restrict__ partials, int max_parts, int heads, int kv_heads, int dk,
-    int dv, int64_t k_stride, int64_t v_stride, int window, int shared_kv) {
+    int dv, int64_t k_stride, int64_t v_stride, int window, int shared_kv, int keep_first, int64_t out_stride) {
   static_assert(NTM / 2 == NSM, "value fragments of shared rows are the key fragments");
   constexpr int QB = 1;
   constexpr bool DECODE = true;
@@ -60,6 +60,8 @@ __global__ __launch_bounds__(64) void ragged_attention_mfma_decode_kernel(
   const int start = seq_start[b], first = seq_first_pos[b];
   const int group = heads / kv_heads;
   int g, k_lo, k_hi, k_begin;   // k_begin: the first key a window still keeps (0 without one)
+  int kept = 0;                 // the sequence's first keys that stay visible in front of the window
+  int jump_from = -1, jump_to = 0;   // the tile walk leaves out what lies between the kept keys and the window
   int head[QB], token[QB], qpos[QB];
   bool valid[QB];
   {
@@ -71,11 +73,26 @@ __global__ __launch_bounds__(64) void ragged_attention_mfma_decode_kernel(
     token[0] = start;
     qpos[0] = first;  // (a decoded token: the sequence brings one)
     k_begin = window > 0 && first - window + 1 > 0 ? first - window + 1 : 0;
+    kept = keep_first < k_begin ? keep_first : k_begin;
     k_lo = blockIdx.x * kPart;
-    if (k_lo > first || k_lo + kPart <= k_begin) return;   // (a partition past the token, or wholly in front of the window)
+    const bool in_window = !(k_lo > first || k_lo + kPart <= k_begin), in_kept = k_lo < kept;
+    if (!in_window && !in_kept) return;   // (a partition past the token, or in front of the window with no kept key)
     k_hi = k_lo + kPart < first + 1 ? k_lo + kPart : first + 1;
-    if (k_lo < k_begin) k_lo = (k_begin / 32) * 32;         // the window's first partition starts at the tile that holds k_begin
+    if (!in_window) k_hi = k_hi < kept ? k_hi : kept;
+    if (k_lo < k_begin) {                 // the window's first partition starts at the tile that holds k_begin ...
+      const int w_lo = (k_begin / 32) * 32;
+      if (!in_kept) {
+        k_lo = w_lo;
+      } else if (in_window) {             // ... behind the tiles of the kept keys, when the partition holds both
+        const int kept_end = ((kept < k_hi ? kept : k_hi) + 31) / 32 * 32;
+        if (kept_end < w_lo) {
+          jump_from = kept_end;
+          jump_to = w_lo;
+        }
+      }
+    }
   }
+  auto next_tile = [&](int p) { return p + 32 == jump_from ? jump_to : p + 32; };
   const int32_t* table = token_table + (int64_t)seq_req[b] * tt_stride;
   const uint16_t* vtr = lds_v + (4 * c + (t >> 2)) * VSTR + (t & 3) * 4;
   const int ns = (dk + 31) / 32, nt = (dv + 15) / 16, nsv = (dv + 31) / 32;
@@ -94,7 +111,7 @@ __global__ __launch_bounds__(64) void ragged_attention_mfma_decode_kernel(
     }
     m_i[qb] = -INFINITY;
     d_i[qb] = 0.f;
-    if (sink && (int)blockIdx.x == k_begin / kPart) {
+    if (sink && (int)blockIdx.x == (kept > 0 ? 0 : k_begin / kPart)) {
       m_i[qb] = to_f32<DT>(sink[head[qb]]) * kLog2e;
       d_i[qb] = 1.0f;
     }
@@ -137,13 +154,14 @@ __global__ __launch_bounds__(64) void ragged_attention_mfma_decode_kernel(
   {
     int64_t ra, rb;
     rows_of(k_lo, ra, rb);
-    rows_of(k_lo + 32, nra, nrb);
+    rows_of(next_tile(k_lo), nra, nrb);
     fetch(k_lo, ra, rb, ka, kb, va, vb);
   }
-  for (int p0 = k_lo; p0 < k_hi; p0 += 32) {
+  for (int p0 = k_lo, p1; p0 < k_hi; p0 = p1) {
+    p1 = next_tile(p0);
     Q4 nka[NSM], nkb[NSM], nva[NTM / 2], nvb[NTM / 2];
-    fetch(p0 + 32, nra, nrb, nka, nkb, nva, nvb);   // (past the range: nothing is read)
-    rows_of(p0 + 64, nra, nrb);
+    fetch(p1, nra, nrb, nka, nkb, nva, nvb);   // (past the range: nothing is read)
+    rows_of(next_tile(p1), nra, nrb);
     Q4 pf_hi[QB], pf_lo[QB];
     float alpha[QB];
     bool moved[QB];   // some column's running maximum moved (wave-uniform): only then the outputs are rescaled
@@ -162,8 +180,8 @@ __global__ __launch_bounds__(64) void ragged_attention_mfma_decode_kernel(
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int k0i = p0 + 4 * c + r, k1i = k0i + 16;
-        sc[r] = (k0i <= qpos[qb] && k0i < k_hi && k0i >= k_begin) ? sa[r] * scale_log2 : -INFINITY;
-        sc[4 + r] = (k1i <= qpos[qb] && k1i < k_hi && k1i >= k_begin) ? sb[r] * scale_log2 : -INFINITY;
+        sc[r] = (k0i <= qpos[qb] && k0i < k_hi && (k0i >= k_begin || k0i < kept)) ? sa[r] * scale_log2 : -INFINITY;
+        sc[4 + r] = (k1i <= qpos[qb] && k1i < k_hi && (k1i >= k_begin || k1i < kept)) ? sb[r] * scale_log2 : -INFINITY;
         mx = fmaxf(mx, fmaxf(sc[r], sc[4 + r]));
       }
       mx = rows_max(mx);
@@ -240,7 +258,7 @@ __global__ __launch_bounds__(64) void ragged_attention_mfma_decode_kernel(
     if (!valid[qb]) continue;
     if (!DECODE || max_parts == 1) {
       const float inv = 1.0f / d_i[qb];
-      uint16_t* o = out + ((int64_t)token[qb] * heads + head[qb]) * dv;
+      uint16_t* o = out + (int64_t)token[qb] * out_stride + (int64_t)head[qb] * dv;
 #pragma unroll
       for (int dt = 0; dt < NTM; ++dt) {
 #pragma unroll
@@ -279,7 +297,7 @@ __global__ __launch_bounds__(256) void ragged_attention_mfma_prefill4_kernel(
     const int32_t* __restrict__ token_table, int64_t tt_stride, const int32_t* __restrict__ seq_req,
     const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_first_pos, const uint16_t* __restrict__ sink,
     float scale_log2, uint16_t* __restrict__ out, int heads, int kv_heads, int dk, int dv, int64_t k_stride, int64_t v_stride,
-    int window, int shared_kv) {
+    int window, int shared_kv, int keep_first, int64_t out_stride) {
   constexpr int KSTR = NSM * 32 + 8, VSTR = NTM * 16 + 8;
   constexpr int KPASS = (32 * NSM * 4 + 255) / 256, VPASS = (32 * NTM * 2 + 255) / 256;  // 16-byte pieces per thread
   __shared__ __attribute__((aligned(16))) uint16_t lds_k[32 * KSTR];
@@ -302,6 +320,13 @@ __global__ __launch_bounds__(256) void ragged_attention_mfma_prefill4_kernel(
   const int k_lo_wg = window > 0 && first + q0 - window + 1 > 0 ? ((first + q0 - window + 1) / 32) * 32 : 0;
   const int k_lo_w = window > 0 && first + qw - window + 1 > 0 ? first + qw - window + 1 : 0;
   const int wlo = window > 0 ? qpos - window + 1 : 0;
+  // the sequence's first `keep_first` keys stay visible in front of a window: their tiles are walked first, then the walk jumps
+  // to the window's first tile (keys in position order, whatever the step looks like)
+  const int kept_wg = keep_first < k_lo_wg ? keep_first : k_lo_wg;
+  const int kept_end = (kept_wg + 31) / 32 * 32;
+  const int k_first_wg = kept_wg > 0 ? 0 : k_lo_wg;
+  const int jump_from = kept_wg > 0 && kept_end < k_lo_wg ? kept_end : -1;
+  auto next_tile = [&](int p) { return p + 32 == jump_from ? k_lo_wg : p + 32; };
   const int32_t* table = token_table + (int64_t)seq_req[b] * tt_stride;
   const int ns = (dk + 31) / 32, nt = (dv + 15) / 16;
   const int kcpr = dk / 8, vcpr = dv / 8;                                  // 16-byte pieces per cache row
@@ -352,13 +377,14 @@ __global__ __launch_bounds__(256) void ragged_attention_mfma_prefill4_kernel(
     const int i = tid + 256 * u, key = i / vcpr, piece = i - key * vcpr;                     \
     if (key < 32) *reinterpret_cast<Q4*>(&lds_v[key * VSTR + 8 * piece]) = vr[u];            \
   }
-  LL_FETCH(k_lo_wg)
+  LL_FETCH(k_first_wg)
   __syncthreads();   // the zero fill is complete
   LL_STAGE()
   __syncthreads();
-  for (int p0 = k_lo_wg; p0 < k_hi; p0 += 32) {
-    if (p0 + 32 < k_hi) { LL_FETCH(p0 + 32) }
-    if (wave_on && p0 < k_hi_w && p0 + 32 > k_lo_w) {
+  for (int p0 = k_first_wg, p1; p0 < k_hi; p0 = p1) {
+    p1 = next_tile(p0);
+    if (p1 < k_hi) { LL_FETCH(p1) }
+    if (wave_on && p0 < k_hi_w && (p0 + 32 > k_lo_w || p0 < keep_first)) {
       f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int s = 0; s < NSM; ++s) {
@@ -374,8 +400,8 @@ __global__ __launch_bounds__(256) void ragged_attention_mfma_prefill4_kernel(
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int k0i = p0 + 4 * c + r, k1i = k0i + 16;
-        sc[r] = (k0i <= qpos && k0i >= wlo) ? sa[r] * scale_log2 : -INFINITY;
-        sc[4 + r] = (k1i <= qpos && k1i >= wlo) ? sb[r] * scale_log2 : -INFINITY;
+        sc[r] = (k0i <= qpos && (k0i >= wlo || k0i < keep_first)) ? sa[r] * scale_log2 : -INFINITY;
+        sc[4 + r] = (k1i <= qpos && (k1i >= wlo || k1i < keep_first)) ? sb[r] * scale_log2 : -INFINITY;
         mx = fmaxf(mx, fmaxf(sc[r], sc[4 + r]));
       }
       mx = rows_max(mx);
@@ -419,14 +445,14 @@ __global__ __launch_bounds__(256) void ragged_attention_mfma_prefill4_kernel(
       }
     }
     __syncthreads();   // everybody has read this tile
-    if (p0 + 32 < k_hi) { LL_STAGE() }
+    if (p1 < k_hi) { LL_STAGE() }
     __syncthreads();
   }
 #undef LL_FETCH
 #undef LL_STAGE
   if (!valid) return;
   const float inv = 1.0f / d_i;
-  uint16_t* o = out + ((int64_t)token * heads + head) * dv;
+  uint16_t* o = out + (int64_t)token * out_stride + (int64_t)head * dv;
 #pragma unroll
   for (int dt = 0; dt < NTM; ++dt) {
 #pragma unroll
@@ -442,23 +468,30 @@ template <int DT>
 __global__ __launch_bounds__(256) void ragged_attention_merge_kernel(const float* __restrict__ partials, int max_parts,
                                                                      const int32_t* __restrict__ seq_first_pos,
                                                                      uint16_t* __restrict__ out, int64_t n, int heads, int dv,
-                                                                     int window) {
+                                                                     int window, int keep_first, int64_t out_stride) {
   const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (w >= n * heads) return;
   const int lane = threadIdx.x & 63;
   const int64_t token = w / heads;
   const int pos = seq_first_pos[token];                // (decoded tokens: token index == sequence index)
   const int parts = pos / kPart + 1;
-  const int p_lo = window > 0 && pos - window + 1 > 0 ? (pos - window + 1) / kPart : 0;   // partitions in front of it wrote nothing
+  const int k_begin = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
+  const int p_lo = k_begin / kPart;   // partitions in front of it wrote nothing, but for those that hold kept first keys
+  const int kept = keep_first < k_begin ? keep_first : k_begin;
+  const int p_kept = (kept + kPart - 1) / kPart;
   const float* src = partials + w * max_parts * (2 + dv);
   float m = -INFINITY;
-  for (int p = p_lo; p < parts; ++p) m = fmaxf(m, src[p * (2 + dv)]);
+  for (int p = 0; p < parts; ++p)
+    if (p >= p_lo || p < p_kept) m = fmaxf(m, src[p * (2 + dv)]);
   float d = 0.f;
-  for (int p = p_lo; p < parts; ++p) d += src[p * (2 + dv) + 1] * exp2f(src[p * (2 + dv)] - m);
+  for (int p = 0; p < parts; ++p)
+    if (p >= p_lo || p < p_kept) d += src[p * (2 + dv) + 1] * exp2f(src[p * (2 + dv)] - m);
+  const int h = (int)(w - token * heads);
   for (int ch = lane; ch < dv; ch += 64) {
     float o = 0.f;
-    for (int p = p_lo; p < parts; ++p) o += src[p * (2 + dv) + 2 + ch] * exp2f(src[p * (2 + dv)] - m);
-    out[w * dv + ch] = from_f32<DT>(o / d);
+    for (int p = 0; p < parts; ++p)
+      if (p >= p_lo || p < p_kept) o += src[p * (2 + dv) + 2 + ch] * exp2f(src[p * (2 + dv)] - m);
+    out[token * out_stride + (int64_t)h * dv + ch] = from_f32<DT>(o / d);
   }
 }
 
@@ -478,9 +511,10 @@ extern "C" int ll_ragged_attention_mfma(const void* q, const void* k_cache, cons
                                         const int32_t* seq_first_pos, const void* sink, float scale, void* out, int64_t n,
                                         int64_t batch, int64_t longest_run, int64_t longest_context, int decode, float* partials,
                                         int64_t heads, int64_t kv_heads, int64_t dk, int64_t dv, int64_t k_stride, int64_t v_stride,
-                                        int64_t window, int dtype, void* stream) {
+                                        int64_t window, int64_t keep_first, int64_t out_stride, int dtype, void* stream) {
   if (!ll_ragged_attention_mfma_supported(dk, dv, dtype)) return dtype == LL_F32 ? LL_ERR_DTYPE : LL_ERR_SHAPE;
   if (k_stride < kv_heads * dk || v_stride < kv_heads * dv || k_stride % 8 || v_stride % 8 || window < 0 || window > 0x7fffffff ||
+      keep_first < 0 || keep_first > 0x7fffffff || out_stride < heads * dv ||
       !ll_aligned16(k_cache) || !ll_aligned16(v_cache) || !ll_aligned16(q))
     return LL_ERR_SHAPE;
   if (n < 0 || batch < 0 || heads < 1 || kv_heads < 1 || heads % kv_heads || heads > 65535 || batch > 65535 || longest_run < 1 ||
@@ -499,7 +533,7 @@ extern "C" int ll_ragged_attention_mfma(const void* q, const void* k_cache, cons
   ragged_attention_mfma_decode_kernel<DT, NS, NT><<<grid, 64, 0, st>>>(                                                      \
       (const uint16_t*)q, (const uint16_t*)k_cache, (const uint16_t*)v_cache, token_table, tt_stride, seq_req, seq_start,    \
       seq_first_pos, (const uint16_t*)sink, scale_log2, (uint16_t*)out, partials, max_parts, (int)heads, (int)kv_heads, (int)dk, \
-      (int)dv, k_stride, v_stride, (int)window, shared_kv)
+      (int)dv, k_stride, v_stride, (int)window, shared_kv, (int)keep_first, out_stride)
 #define CALL(DT)                                         \
   if (dk <= 64 && dv <= 64) { CALL_D(DT, 2, 4); }        \
   else if (dk <= 128 && dv <= 128) { CALL_D(DT, 4, 8); } \
@@ -510,7 +544,7 @@ extern "C" int ll_ragged_attention_mfma(const void* q, const void* k_cache, cons
   ragged_attention_mfma_prefill4_kernel<DT, NS, NT><<<grid4, 256, 0, st>>>(                                                 \
       (const uint16_t*)q, (const uint16_t*)k_cache, (const uint16_t*)v_cache, token_table, tt_stride, seq_req, seq_start,   \
       seq_first_pos, (const uint16_t*)sink, scale_log2, (uint16_t*)out, (int)heads, (int)kv_heads, (int)dk, (int)dv, k_stride,   \
-      v_stride, (int)window, shared_kv)
+      v_stride, (int)window, shared_kv, (int)keep_first, out_stride)
 #define CALL_P(DT)                                       \
   if (dk <= 64 && dv <= 64) { CALL_4(DT, 2, 4); }        \
   else if (dk <= 128 && dv <= 128) { CALL_4(DT, 4, 8); } \
@@ -527,10 +561,10 @@ extern "C" int ll_ragged_attention_mfma(const void* q, const void* k_cache, cons
     const int64_t waves = n * heads;
     if (dtype == LL_F16)
       ragged_attention_merge_kernel<LL_F16><<<dim3((unsigned)((waves + 3) / 4)), 256, 0, st>>>(partials, max_parts, seq_first_pos,
-                                                                                            (uint16_t*)out, n, (int)heads, (int)dv, (int)window);
+                                                                                            (uint16_t*)out, n, (int)heads, (int)dv, (int)window, (int)keep_first, out_stride);
     else
       ragged_attention_merge_kernel<LL_BF16><<<dim3((unsigned)((waves + 3) / 4)), 256, 0, st>>>(partials, max_parts, seq_first_pos,
-                                                                                             (uint16_t*)out, n, (int)heads, (int)dv, (int)window);
+                                                                                             (uint16_t*)out, n, (int)heads, (int)dv, (int)window, (int)keep_first, out_stride);
   }
   return LL_LAUNCH_CHECK();
 }

@@ -2,7 +2,10 @@
 // prompt, or one decoded token) with a 32-bit residual stream:
 //
 //   ll_add_rmsnorm_shift   residual add (fp32) + RMS norm (fp32) + optional token shift against the previous token's normed
-//                          row (carried per sequence in a state slot) -> activations in the storage dtype
+//                          row (carried per sequence in a state slot) -> activations in the storage dtype; the update may come
+//                          as one row plus several part rows per token (sublayers that ran side by side, experts' slots)
+//   ll_embed_pair          token embedding times a scale plus a row of a hashed (previous token, token) table -> fp32 residual;
+//                          the previous token of a run's first token is carried per sequence in a state slot
 //   ll_xielu               the xIELU activation with its two learned numbers
 //   ll_cast_pair / ll_residual_set   the two ends of a projection over [x ; x0] that re-enters the residual stream
 //   ll_gated_linear_scan   per-head linear recurrence S_t = diag(f_t) S_(t-1) + (1 - f_t) v_t^T, o_t = S_t^T q_t with a
@@ -43,6 +46,18 @@ __device__ __forceinline__ float block_sum256(float v, float* lds4) {
   return ((lds4[0] + lds4[1]) + lds4[2]) + lds4[3];
 }
 
+// the update of row t at element i: delta row + the row's parts in order (either may be absent), fp32
+template <int DT>
+__device__ __forceinline__ float update_at(const void* delta, const void* parts, int num_parts, int64_t t, int width, int i) {
+  float u = delta ? ldv<DT>(delta, t * width + i) : 0.f;
+  if (parts) {
+    float p = ldv<DT>(parts, (t * num_parts) * width + i);
+    for (int k = 1; k < num_parts; ++k) p += ldv<DT>(parts, (t * num_parts + k) * width + i);
+    u = delta ? u + p : p;
+  }
+  return u;
+}
+
 // One workgroup per token.  s = x_in + delta (fp32; written to x_out when delta is given), h = s / sqrt(mean(s^2) + eps) * w,
 // y = h + (h_prev - h) * shift, h_prev = the same h of the previous token of the sequence: recomputed from the previous row
 // when that token is part of this step, read from the sequence's state slot when the run starts inside the sequence, zero
@@ -53,15 +68,17 @@ __global__ __launch_bounds__(256) void add_rmsnorm_shift_kernel(
     const float* __restrict__ x_in, const void* __restrict__ delta, float* __restrict__ x_out, const void* __restrict__ weight,
     const void* __restrict__ shift, void* __restrict__ y, int64_t n, int width, float eps, const int32_t* __restrict__ tok_seq,
     const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_first_pos, const int32_t* __restrict__ seq_slot,
-    const int32_t* __restrict__ seq_parity, float* __restrict__ state, int64_t state_half) {
+    const int32_t* __restrict__ seq_parity, float* __restrict__ state, int64_t state_half, const void* __restrict__ parts,
+    int num_parts, float out_scale) {
   __shared__ float red[4];
   const int64_t t = blockIdx.x;
   const int tid = threadIdx.x;
   const float* xr = x_in + t * width;
+  const bool upd = delta || parts;
   float ss = 0.f;
   for (int i = tid; i < width; i += 256) {
     float s = xr[i];
-    if (delta) s += ldv<DT>(delta, t * width + i);
+    if (upd) s += update_at<DT>(delta, parts, num_parts, t, width, i);
     ss += s * s;
   }
   ss = block_sum256(ss, red);
@@ -79,7 +96,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_shift_kernel(
       float sp = 0.f;
       for (int i = tid; i < width; i += 256) {
         float s = pr[i];
-        if (delta) s += ldv<DT>(delta, (t - 1) * width + i);
+        if (upd) s += update_at<DT>(delta, parts, num_parts, t - 1, width, i);
         sp += s * s;
       }
       sp = block_sum256(sp, red);
@@ -96,8 +113,8 @@ __global__ __launch_bounds__(256) void add_rmsnorm_shift_kernel(
     keep = state + (int64_t)(1 - seq_parity[b]) * state_half + (int64_t)seq_slot[b] * width;
   for (int i = tid; i < width; i += 256) {
     float s = xr[i];
-    if (delta) {
-      s += ldv<DT>(delta, t * width + i);
+    if (upd) {
+      s += update_at<DT>(delta, parts, num_parts, t, width, i);
       x_out[t * width + i] = s;
     }
     const float w = ldv<DT>(weight, i);
@@ -107,7 +124,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_shift_kernel(
       float hp = 0.f;
       if (mode == 1) {
         float s1 = x_in[(t - 1) * width + i];
-        if (delta) s1 += ldv<DT>(delta, (t - 1) * width + i);
+        if (upd) s1 += update_at<DT>(delta, parts, num_parts, t - 1, width, i);
         hp = s1 * inv_prev * w;
       } else if (mode == 2) {
         hp = prev_state[i];
@@ -115,7 +132,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_shift_kernel(
       out = h + (hp - h) * ldv<DT>(shift, i);
       if (keep) keep[i] = h;
     }
-    stv<DT>(y, t * width + i, out);
+    stv<DT>(y, t * width + i, out * out_scale);
   }
 }
 
@@ -145,16 +162,35 @@ __device__ __forceinline__ void st4(void* p, int64_t i, f32x4 v) {
   }
 }
 
+// update_at for four elements at i (a multiple of 4): the same sums in the same order
+template <int DT>
+__device__ __forceinline__ f32x4 update4(const void* delta, const void* parts, int num_parts, int64_t t, int width, int i) {
+  f32x4 u = {0.f, 0.f, 0.f, 0.f};
+  if (delta) u = ld4<DT>(delta, t * width + i);
+  if (parts) {
+    f32x4 p = ld4<DT>(parts, (t * num_parts) * width + i);
+    for (int k = 1; k < num_parts; ++k) {
+      const f32x4 q = ld4<DT>(parts, (t * num_parts + k) * width + i);
+      p[0] += q[0]; p[1] += q[1]; p[2] += q[2]; p[3] += q[3];
+    }
+    if (delta) { u[0] += p[0]; u[1] += p[1]; u[2] += p[2]; u[3] += p[3]; }
+    else u = p;
+  }
+  return u;
+}
+
 template <int DT, int NV>
 __global__ __launch_bounds__(256) void add_rmsnorm_shift_vec_kernel(
     const float* __restrict__ x_in, const void* __restrict__ delta, float* __restrict__ x_out, const void* __restrict__ weight,
     const void* __restrict__ shift, void* __restrict__ y, int64_t n, int width, float eps, const int32_t* __restrict__ tok_seq,
     const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_first_pos, const int32_t* __restrict__ seq_slot,
-    const int32_t* __restrict__ seq_parity, float* __restrict__ state, int64_t state_half) {
+    const int32_t* __restrict__ seq_parity, float* __restrict__ state, int64_t state_half, const void* __restrict__ parts,
+    int num_parts, float out_scale) {
   __shared__ float red[4];
   const int64_t t = blockIdx.x;
   const int tid = threadIdx.x;
   f32x4 s[NV], sp[NV];
+  const bool upd = delta || parts;
   float ss = 0.f;
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
@@ -162,8 +198,8 @@ __global__ __launch_bounds__(256) void add_rmsnorm_shift_vec_kernel(
     s[j] = f32x4{0.f, 0.f, 0.f, 0.f};
     if (i < width) {
       s[j] = *reinterpret_cast<const f32x4*>(x_in + t * width + i);
-      if (delta) {
-        const f32x4 d = ld4<DT>(delta, t * width + i);
+      if (upd) {
+        const f32x4 d = update4<DT>(delta, parts, num_parts, t, width, i);
         s[j][0] += d[0]; s[j][1] += d[1]; s[j][2] += d[2]; s[j][3] += d[3];
       }
       // (element order i, i + 1, ..: the plain form adds the same values thread by thread in steps of 256 -- the per-thread
@@ -187,8 +223,8 @@ __global__ __launch_bounds__(256) void add_rmsnorm_shift_vec_kernel(
         sp[j] = f32x4{0.f, 0.f, 0.f, 0.f};
         if (i < width) {
           sp[j] = *reinterpret_cast<const f32x4*>(x_in + (t - 1) * width + i);
-          if (delta) {
-            const f32x4 d = ld4<DT>(delta, (t - 1) * width + i);
+          if (upd) {
+            const f32x4 d = update4<DT>(delta, parts, num_parts, t - 1, width, i);
             sp[j][0] += d[0]; sp[j][1] += d[1]; sp[j][2] += d[2]; sp[j][3] += d[3];
           }
           q += sp[j][0] * sp[j][0]; q += sp[j][1] * sp[j][1]; q += sp[j][2] * sp[j][2]; q += sp[j][3] * sp[j][3];
@@ -210,7 +246,7 @@ __global__ __launch_bounds__(256) void add_rmsnorm_shift_vec_kernel(
   for (int j = 0; j < NV; ++j) {
     const int i = (tid + 256 * j) * 4;
     if (i < width) {
-      if (delta) *reinterpret_cast<f32x4*>(x_out + t * width + i) = s[j];
+      if (upd) *reinterpret_cast<f32x4*>(x_out + t * width + i) = s[j];
       const f32x4 w = ld4<DT>(weight, i);
       f32x4 h, o;
 #pragma unroll
@@ -229,6 +265,8 @@ __global__ __launch_bounds__(256) void add_rmsnorm_shift_vec_kernel(
         for (int e = 0; e < 4; ++e) o[e] = h[e] + (hp[e] - h[e]) * mu[e];
         if (keep) *reinterpret_cast<f32x4*>(keep + i) = h;
       }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] *= out_scale;
       st4<DT>(y, t * width + i, o);
     }
   }
@@ -301,6 +339,36 @@ __global__ __launch_bounds__(256) void residual_set_kernel(float* __restrict__ x
     float v = ldv<DT>(y, i);
     if (bias) v += ldv<DT>(bias, i % width);
     x[i] = v;
+  }
+}
+
+// One workgroup per token: x = embed[token] * scale + pair[row], row = (previous token * mul_prev + token * mul_cur) mod buckets,
+// or row `buckets` (the table's last) for a sequence's first token.  The previous token of a run's first token comes from the
+// sequence's state slot (half seq_parity is read); a run's last token leaves itself in the other half.  pair == NULL: no table.
+template <int DT>
+__global__ __launch_bounds__(256) void embed_pair_kernel(
+    float* __restrict__ x, const int32_t* __restrict__ tokens, const void* __restrict__ embed, int64_t vocab, float scale,
+    const void* __restrict__ pair, int64_t buckets, int64_t mul_prev, int64_t mul_cur, int width,
+    const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_first_pos,
+    const int32_t* __restrict__ seq_slot, const int32_t* __restrict__ seq_parity, int32_t* __restrict__ prev_state,
+    int64_t state_half) {
+  const int64_t t = blockIdx.x;
+  int64_t tok = tokens[t];
+  tok = tok < 0 ? 0 : tok >= vocab ? vocab - 1 : tok;   // (the host refuses ids outside the table; never read past it)
+  int64_t row = buckets;
+  if (pair) {
+    const int b = tok_seq[t];
+    int64_t prev = -1;
+    if (t > seq_start[b]) prev = tokens[t - 1];
+    else if (seq_first_pos[b] > 0) prev = prev_state[(int64_t)seq_parity[b] * state_half + seq_slot[b]];
+    if (prev >= 0) row = (prev * mul_prev + tok * mul_cur) % buckets;
+    if (t == seq_start[b + 1] - 1 && threadIdx.x == 0)
+      prev_state[(int64_t)(1 - seq_parity[b]) * state_half + seq_slot[b]] = (int32_t)tok;
+  }
+  for (int i = threadIdx.x; i < width; i += 256) {
+    float v = ldv<DT>(embed, tok * width + i) * scale;
+    if (pair) v += ldv<DT>(pair, row * width + i);
+    x[t * width + i] = v;
   }
 }
 
@@ -630,16 +698,19 @@ __global__ __launch_bounds__(256) void mingru_carry_kernel(int width, const int3
 extern "C" int ll_add_rmsnorm_shift(const float* x_in, const void* delta, float* x_out, const void* weight, const void* shift,
                                     void* y, int64_t n, int64_t width, float eps, const int32_t* tok_seq,
                                     const int32_t* seq_start, const int32_t* seq_first_pos, const int32_t* seq_slot,
-                                    const int32_t* seq_parity, float* state, int64_t state_half, int dtype, void* stream) {
+                                    const int32_t* seq_parity, float* state, int64_t state_half, const void* parts,
+                                    int64_t num_parts, float out_scale, int dtype, void* stream) {
   if (dtype != LL_F16 && dtype != LL_BF16 && dtype != LL_F32) return LL_ERR_DTYPE;
-  if (n < 0 || width < 1 || width > (1 << 20)) return LL_ERR_SHAPE;
+  if (n < 0 || width < 1 || width > (1 << 20) || num_parts < 0 || num_parts > 64 || (parts && num_parts < 1)) return LL_ERR_SHAPE;
   if (n == 0) return LL_OK;
-  if (!x_in || !weight || !y || (delta && !x_out)) return LL_ERR_ARG;
-  if (delta && x_out == x_in && shift) return LL_ERR_ARG;  // the previous row is re-read: it must still hold the old sum
+  if (!x_in || !weight || !y || ((delta || parts) && !x_out)) return LL_ERR_ARG;
+  if ((delta || parts) && x_out == x_in && shift) return LL_ERR_ARG;  // the previous row is re-read: it must still hold the old sum
   if (shift && (!tok_seq || !seq_start || !seq_first_pos || !seq_slot || !seq_parity || !state)) return LL_ERR_ARG;
 #define LL_NORM_ARGS \
-  x_in, delta, x_out, weight, shift, y, n, (int)width, eps, tok_seq, seq_start, seq_first_pos, seq_slot, seq_parity, state, state_half
-  const bool vec = width % 4 == 0 && width <= 4096 && ll_aligned16(x_in) && (!delta || (ll_aligned16(delta) && ll_aligned16(x_out))) &&
+  x_in, delta, x_out, weight, shift, y, n, (int)width, eps, tok_seq, seq_start, seq_first_pos, seq_slot, seq_parity, state, state_half, \
+      parts, (int)num_parts, out_scale
+  const bool vec = width % 4 == 0 && width <= 4096 && ll_aligned16(x_in) && (!delta || ll_aligned16(delta)) &&
+                   (!parts || ll_aligned16(parts)) && (!(delta || parts) || ll_aligned16(x_out)) &&
                    ll_aligned16(weight) && ll_aligned16(y) && (!shift || (ll_aligned16(shift) && ll_aligned16(state)));
   const dim3 grid((unsigned)n);
   hipStream_t st = (hipStream_t)stream;
@@ -687,6 +758,24 @@ extern "C" int ll_residual_set(float* x, const void* y, const void* bias, int64_
   if (n == 0) return LL_OK;
   if (!x || !y) return LL_ERR_ARG;
 #define CALL(DT) residual_set_kernel<DT><<<dim3(flat_grid(n * width)), 256, 0, (hipStream_t)stream>>>(x, y, bias, n, (int)width)
+  LL_BY_DTYPE(dtype, CALL);
+#undef CALL
+  return LL_LAUNCH_CHECK();
+}
+
+extern "C" int ll_embed_pair(float* x, const int32_t* tokens, const void* embed, int64_t vocab, float scale, const void* pair,
+                             int64_t buckets, int64_t mul_prev, int64_t mul_cur, int64_t n, int64_t width, const int32_t* tok_seq,
+                             const int32_t* seq_start, const int32_t* seq_first_pos, const int32_t* seq_slot,
+                             const int32_t* seq_parity, int32_t* prev_state, int64_t state_half, int dtype, void* stream) {
+  if (dtype != LL_F16 && dtype != LL_BF16 && dtype != LL_F32) return LL_ERR_DTYPE;
+  if (n < 0 || width < 1 || width > (1 << 20) || vocab < 1 || (pair && (buckets < 1 || mul_prev < 0 || mul_cur < 0))) return LL_ERR_SHAPE;
+  if (n == 0) return LL_OK;
+  if (!x || !tokens || !embed) return LL_ERR_ARG;
+  if (pair && (!tok_seq || !seq_start || !seq_first_pos || !seq_slot || !seq_parity || !prev_state)) return LL_ERR_ARG;
+#define CALL(DT)                                                                                                              \
+  embed_pair_kernel<DT><<<dim3((unsigned)n), 256, 0, (hipStream_t)stream>>>(x, tokens, embed, vocab, scale, pair, buckets, mul_prev, \
+                                                                            mul_cur, (int)width, tok_seq, seq_start, seq_first_pos, \
+                                                                            seq_slot, seq_parity, prev_state, state_half)
   LL_BY_DTYPE(dtype, CALL);
 #undef CALL
   return LL_LAUNCH_CHECK();

@@ -97,23 +97,39 @@ class PagedStateCache(PagedKVPool):
     """Cache of a model whose layer RUNS differ in what they keep per sequence (a layer that runs several times in a forward
     pass keeps one set per run): attention runs own ``(K [rows, kv_heads, dk], V [rows, kv_heads, dv])`` in the block pool --
     key and value widths may differ --, latent-attention runs one row ``[latent | rotated key part]`` per token, recurrent runs own a fixed-size fp32 state ``[slots, heads, dk, dv]``, and any run may
-    own a token-shift row pair ``[2, slots, width]`` (double-buffered by the sequence's parity).  One block allocator, one
+    own a token-shift row pair ``[2, slots, width]`` (double-buffered by the sequence's parity).  An attention run with a short
+    convolution in front of it carries the projected rows of a sequence's last positions, ``[2, slots, taps - 1, channels]``,
+    double-buffered the same way; a run whose values are blended with those of an earlier run names that run in
+    ``value_source``; a model whose input depends on the previous token keeps it per sequence in ``prev_token [2, slots]``.  One block allocator, one
     block table and one per-token row table serve all attention runs; a sequence's slot is its row of those tables, so blocks
     and slots are handed out and given back together.  Fixed-size state is never cleared: the kernels start a sequence whose
     run begins at position 0 from zeros, whatever an earlier owner of the slot left."""
 
-    def __init__(self, runs, num_blocks: int, block_size: int, device, max_requests: int, max_seq_len: int, dtype):
+    def __init__(self, runs, num_blocks: int, block_size: int, device, max_requests: int, max_seq_len: int, dtype,
+                 previous_token: bool = False):
         """``runs``: one mapping per layer run: ``{"kind": "attention", "kv_heads", "dk", "dv"}``, ``{"kind": "latent", "rank",
-        "rot"}`` or ``{"kind": "recurrent", "heads", "dk", "dv"}``, each with an optional ``"shift_width"``."""
+        "rot"}`` or ``{"kind": "recurrent", "heads", "dk", "dv"}``, each with an optional ``"shift_width"``; attention runs may
+        add ``"conv_taps"`` / ``"conv_channels"`` (rows carried for a convolution of that many taps) and ``"value_mix": True``
+        (the first such run is the value source of the later ones).  ``previous_token``: keep each sequence's last token."""
         self.runs = [dict(r) for r in runs]
         self.dtype = dtype
+        self.prev_token = torch.zeros(2, max_requests, dtype=torch.int32, device=device) if previous_token else None
         super().__init__(len(self.runs), num_blocks, block_size, 1, 1, device, max_requests, max_seq_len, dtype)
 
     def _make_buffers(self, num_layers, num_kv_heads, head_dim, dtype):
         dev, slots = self.device, self.max_requests
-        self.recurrent, self.shift = [], []
+        self.recurrent, self.shift, self.conv, self.value_source = [], [], [], []
         buffers = []
-        for r in self.runs:
+        first_mix = None
+        for index, r in enumerate(self.runs):
+            taps = int(r.get("conv_taps", 0)) if r["kind"] == "attention" else 0
+            self.conv.append(torch.zeros(2, slots, taps - 1, int(r["conv_channels"]), dtype=dtype, device=dev) if taps > 1 else None)
+            mixes = r["kind"] == "attention" and bool(r.get("value_mix"))
+            self.value_source.append(first_mix if mixes else None)
+            if mixes and first_mix is None:
+                first_mix = index
+            elif mixes and (self.runs[first_mix]["kv_heads"], self.runs[first_mix]["dv"]) != (r["kv_heads"], r["dv"]):
+                raise ValueError(f"layer run {index} blends its values with those of run {first_mix}, whose shape differs")
             if r["kind"] == "attention":
                 buffers.append((torch.zeros(self.max_tokens, r["kv_heads"], r["dk"], dtype=dtype, device=dev),
                                 torch.zeros(self.max_tokens, r["kv_heads"], r["dv"], dtype=dtype, device=dev)))
@@ -140,7 +156,7 @@ class PagedStateCache(PagedKVPool):
 
     def state_bytes(self) -> int:
         total, seen = 0, set()
-        for group in (self.kv_buffer, self.recurrent, self.shift):
+        for group in (self.kv_buffer, self.recurrent, self.shift, self.conv, [self.prev_token]):
             for t in group:
                 for u in (t if isinstance(t, tuple) else (t,)):
                     if u is not None and u.untyped_storage().data_ptr() not in seen:   # (a view of counted rows adds nothing)

@@ -70,7 +70,8 @@ class RaggedRunner:
         self.max_seq_len = -(-self.max_seq_len // block_size) * block_size
         self.max_requests = max_requests
         self.cache = PagedStateCache(model.cache_runs(), blocks + 1, block_size, self.device, max_requests, self.max_seq_len,
-                                     model.dtype)
+                                     model.dtype, previous_token=bool(getattr(model, "needs_previous_token", False)))
+        self.vocab_size = int(getattr(getattr(model, "geo", None), "vocab_size", 0))
         self.token_table = torch.zeros(max_requests, self.max_seq_len, dtype=torch.int32, device=self.device)
         self.total_blocks = blocks
         self._free_slots = list(range(max_requests))
@@ -126,6 +127,8 @@ class RaggedRunner:
         counts = [len(t) for _, t in entries]
         if min(counts) < 1:
             raise ValueError("every entry brings at least one token")
+        if self.vocab_size and not all(0 <= int(t) < self.vocab_size for _, toks in entries for t in toks):
+            raise ValueError(f"token ids lie in 0 .. {self.vocab_size - 1}")
         first = [self._len[s] for s in slots]
         new_len = [f + c for f, c in zip(first, counts)]
         if max(new_len) > self.max_seq_len:

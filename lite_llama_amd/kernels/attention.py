@@ -310,12 +310,63 @@ def qk_norm_cache(qkv, heads: int, kv_heads: int, dk: int, dv: int, q_weight, k_
 
 
 @torch.no_grad()
-def ragged_attention(q, k_cache, v_cache, scale: float, step, token_table, sink=None, window: int = 0):
+def conv_rope_cache(qkv, heads: int, kv_heads: int, dk: int, dv: int, step, k_cache, v_cache, *, bias=None, conv_weight=None,
+                    conv_state=None, freq=None, pairs: int = 0, amp: float = 1.0, unit_norm: bool = False, eps: float = 0.0,
+                    v_source=None, v_blend=None):
+    """Fused projection rows ``[q | k | v]`` -> queries ``[n, heads, dk]``; keys and values land in the cache rows
+    ``step.select``.  Channel by channel, in fp32: ``+ bias``; a causal convolution over the sequence's positions with
+    ``conv_weight [channels, taps]`` (``y_t = sum_j w[:, j] u_(t - taps + 1 + j)``, zeros in front of position 0), the raw rows of
+    a sequence's last ``taps - 1`` positions carried in ``conv_state [2, slots, taps - 1, channels]`` (the half named by the
+    sequence's parity is read, the other written); entry pairs ``(2i, 2i + 1)``, ``i < pairs``, of every q / k head rotated by
+    ``position * freq[i]`` with cos / sin times ``amp``; q / k heads divided by ``sqrt(mean + eps)`` when ``unit_norm``; values
+    become ``(1 - b) v + b v_source[select]`` when ``v_source [rows, kv_heads, dv]`` (another layer's value cache) and the
+    one-element tensor ``v_blend`` are given."""
+    L.require_cuda(qkv, k_cache, v_cache, bias, conv_weight, conv_state, freq, v_source, v_blend)
+    n, dt = qkv.shape[0], qkv.dtype
+    channels = (heads + kv_heads) * dk + kv_heads * dv
+    if qkv.dim() != 2 or qkv.stride(1) != 1 or qkv.shape[1] < channels or step.num_tokens != n:
+        raise ValueError("conv_rope_cache: rows hold [q | k | v] of the step's tokens")
+    if k_cache.dtype != dt or v_cache.dtype != dt or tuple(k_cache.shape[1:]) != (kv_heads, dk) \
+            or tuple(v_cache.shape[1:]) != (kv_heads, dv) or not (k_cache.is_contiguous() and v_cache.is_contiguous()):
+        raise ValueError("conv_rope_cache: caches are contiguous [rows, kv_heads, dk] / [rows, kv_heads, dv] in the rows' dtype")
+    if bias is not None and (bias.dtype != dt or bias.numel() != channels or not bias.is_contiguous()):
+        raise ValueError("conv_rope_cache: one bias per channel, in the rows' dtype")
+    taps = 0
+    if conv_weight is not None:
+        if conv_weight.dtype != dt or conv_weight.dim() != 2 or conv_weight.shape[0] != channels or not conv_weight.is_contiguous():
+            raise ValueError("conv_rope_cache: convolution weights are [channels, taps] in the rows' dtype")
+        taps = conv_weight.shape[1]
+        if taps > 1 and (conv_state is None or conv_state.dtype != dt or conv_state.dim() != 4 or conv_state.shape[0] != 2
+                         or tuple(conv_state.shape[2:]) != (taps - 1, channels) or not conv_state.is_contiguous()):
+            raise ValueError("conv_rope_cache: the carried rows are [2, slots, taps - 1, channels] in the rows' dtype")
+    if pairs and (freq is None or freq.dtype != torch.float32 or freq.numel() < pairs or not freq.is_contiguous() or 2 * pairs > dk):
+        raise ValueError("conv_rope_cache: fp32 frequencies, one per rotated pair of a head")
+    if v_source is not None and (v_blend is None or v_blend.dtype != dt or v_blend.numel() != 1 or v_source.dtype != dt
+                                 or tuple(v_source.shape[1:]) != (kv_heads, dv) or not v_source.is_contiguous()
+                                 or v_source.shape[0] != v_cache.shape[0]):
+        raise ValueError("conv_rope_cache: the blended values are another cache of this one's shape, with a one-element weight")
+    q = torch.empty(n, heads, dk, dtype=dt, device=qkv.device)
+    half = conv_state[0].numel() if (conv_state is not None and taps > 1) else 0
+    L.check(L.lib().ll_conv_rope_cache(
+        qkv.data_ptr(), qkv.stride(0), L.ptr(bias), L.ptr(conv_weight), taps, L.ptr(conv_state) if taps > 1 else 0, half,
+        L.ptr(freq) if pairs else 0, int(pairs), float(amp), 1 if unit_norm else 0, float(eps), L.ptr(v_source),
+        v_source.stride(0) if v_source is not None else 0, L.ptr(v_blend) if v_source is not None else 0, step.tok_seq.data_ptr(),
+        step.tok_pos.data_ptr(), step.select.data_ptr(), step.seq_start.data_ptr(), step.seq_first_pos.data_ptr(),
+        step.seq_slot.data_ptr(), step.seq_parity.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), n, heads,
+        kv_heads, dk, dv, L.dtype_code(dt), L.stream_ptr()), "conv_rope_cache")
+    return q
+
+
+@torch.no_grad()
+def ragged_attention(q, k_cache, v_cache, scale: float, step, token_table, sink=None, window: int = 0, keep_first: int = 0,
+                     out=None):
     """Causal softmax attention of every token of a ragged step against positions ``0 .. its own`` of its sequence, keys and
     values read through ``token_table[request][position]``; ``sink [heads]`` adds ``exp(sink_h)`` to each head's denominator;
-    ``window > 0`` keeps the last ``window`` positions (the token's own included).  ``k_cache [rows, kv_heads, dk]`` /
+    ``window > 0`` keeps the last ``window`` positions (the token's own included) and, besides them, the sequence's first
+    ``keep_first`` positions.  ``k_cache [rows, kv_heads, dk]`` /
     ``v_cache [rows, kv_heads, dv]`` may be row-strided views (the values of a latent cache are a column range of its key
-    rows).  Scores, weights and the output sum are fp32.  Returns ``[n, heads * dv]``."""
+    rows).  Scores, weights and the output sum are fp32.  Returns ``[n, heads * dv]`` (``out``: a view of that shape with a
+    unit inner stride, e.g. a column range of the next projection's input)."""
     L.require_cuda(q, k_cache, v_cache, token_table)
     n, heads, dk = q.shape
     kv_heads, dv = v_cache.shape[1], v_cache.shape[2]
@@ -332,7 +383,13 @@ def ragged_attention(q, k_cache, v_cache, scale: float, step, token_table, sink=
     if step.num_tokens != n:
         raise ValueError("ragged_attention: the step describes another number of tokens")
     ks, vs = k_cache.stride(0), v_cache.stride(0)
-    out = torch.empty(n, heads * dv, dtype=dt, device=q.device)
+    if out is None:
+        out = torch.empty(n, heads * dv, dtype=dt, device=q.device)
+    elif out.dtype != dt or tuple(out.shape) != (n, heads * dv) or out.stride(1) != 1 or not out.is_cuda:
+        raise ValueError("ragged_attention: out is [n, heads * dv] in the queries' dtype with a unit inner stride")
+    os_ = max(out.stride(0), heads * dv) if n <= 1 else out.stride(0)
+    if window <= 0:
+        keep_first = 0
     if (step.longest_run and step.longest_context and L.has("ll_ragged_attention_mfma") and not os.environ.get("LL_RAGGED_ATTN_VALU")
             and L.lib().ll_ragged_attention_mfma_supported(dk, dv, L.dtype_code(dt)) and ks % 8 == 0 and vs % 8 == 0
             and k_cache.data_ptr() % 16 == 0 and v_cache.data_ptr() % 16 == 0):
@@ -345,12 +402,13 @@ def ragged_attention(q, k_cache, v_cache, scale: float, step, token_table, sink=
             q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), token_table.data_ptr(), token_table.stride(0),
             step.seq_req.data_ptr(), step.seq_start.data_ptr(), step.seq_first_pos.data_ptr(), L.ptr(sink), float(scale),
             out.data_ptr(), n, step.num_seqs, step.longest_run, step.longest_context, 1 if decode else 0, L.ptr(scratch), heads,
-            kv_heads, dk, dv, ks, vs, int(window), L.dtype_code(dt), L.stream_ptr()), "ragged_attention_mfma")
+            kv_heads, dk, dv, ks, vs, int(window), int(keep_first), os_, L.dtype_code(dt), L.stream_ptr()), "ragged_attention_mfma")
         return out
     L.check(L.lib().ll_ragged_attention(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), token_table.data_ptr(),
                                         token_table.stride(0), step.seq_req.data_ptr(), step.tok_seq.data_ptr(),
                                         step.tok_pos.data_ptr(), L.ptr(sink), float(scale), out.data_ptr(), n, heads, kv_heads, dk,
-                                        dv, ks, vs, int(window), L.dtype_code(dt), L.stream_ptr()), "ragged_attention")
+                                        dv, ks, vs, int(window), int(keep_first), os_, L.dtype_code(dt), L.stream_ptr()),
+            "ragged_attention")
     return out
 
 

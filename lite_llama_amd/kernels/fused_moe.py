@@ -251,12 +251,13 @@ def moe_router(x: torch.Tensor, gate_weight: torch.Tensor, top_k: int, norm_topk
 # ------------------------------------------------------------------------------------- #
 @torch.no_grad()
 def group_router(h: torch.Tensor, router_weight: torch.Tensor, top: int, group_count: int = 1, group_keep: int = 1,
-                 route_scale: float = 1.0, extra_weight: torch.Tensor | None = None):
+                 route_scale: float = 1.0, extra_weight: torch.Tensor | None = None, scoring: str = "sigmoid"):
     """``scores = sigmoid(router_weight h)`` in fp32 (``h`` in its storage dtype); the experts form ``group_count`` equal groups
     of neighbours, a group's score is the sum of its two best, the best ``group_keep`` groups stay eligible; the ``top`` best
     eligible experts are chosen.  Returns ``(ids int32 [n, top], weights fp32 [n, top], extra)``: weights = chosen scores /
     (their sum + 1e-20) * ``route_scale``, slot k = the k-th best; ``extra`` fp32 ``[n]`` = ``sigmoid(extra_weight . h)`` when a
-    further weight row is given (the scale of a shared expert), else ``None``."""
+    further weight row is given (the scale of a shared expert), else ``None``.  ``scoring="softmax_chosen"``: no sigmoid and no
+    groups -- the ``top`` largest logits are chosen and the weights are the softmax over the chosen logits alone."""
     L.require_cuda(h, router_weight, extra_weight)
     n, width = h.shape
     experts = router_weight.shape[0]
@@ -269,7 +270,8 @@ def group_router(h: torch.Tensor, router_weight: torch.Tensor, top: int, group_c
     extra = torch.empty(n, dtype=torch.float32, device=h.device) if extra_weight is not None else None
     logits = torch.empty(n, experts + (1 if extra_weight is not None else 0), dtype=torch.float32, device=h.device)
     L.check(L.lib().ll_group_router(h.data_ptr(), h.stride(0), router_weight.data_ptr(), L.ptr(extra_weight), n, width, experts,
-                                    int(top), int(group_count), int(group_keep), float(route_scale), ids.data_ptr(),
+                                    int(top), int(group_count), int(group_keep), float(route_scale),
+                                    {"sigmoid": 0, "softmax_chosen": 1}[scoring], ids.data_ptr(),
                                     weights.data_ptr(), L.ptr(extra), logits.data_ptr(), L.dtype_code(h.dtype), L.stream_ptr()),
             "group_router")
     return ids, weights, extra

@@ -350,20 +350,51 @@ def rope_and_cache(q, kv, cos, sin, batch_size, seq_len, select_index, kv_buffer
 # ------------------------------------------------------------------------------------- #
 # 32-bit residual stream over ragged steps (csrc/seq_mix.hip)
 # ------------------------------------------------------------------------------------- #
+class SummedUpdate:
+    """The results of sublayers that read the same input and have not entered the residual stream yet: ``row [n, width]`` (or
+    ``None``) plus ``parts [n, k, width]`` (or ``None``: the k experts a token chose), all added in fp32 by the next norm
+    launch: ``x + (row + (part_0 + part_1 + ..))``."""
+
+    __slots__ = ("row", "parts")
+
+    def __init__(self, row=None, parts=None):
+        if row is None and parts is None:
+            raise ValueError("SummedUpdate: nothing to add")
+        self.row, self.parts = row, parts
+
+    def rows(self, index: torch.Tensor) -> "SummedUpdate":
+        """The update of the listed tokens only."""
+        pick = lambda t: None if t is None else t[index].contiguous()  # noqa: E731
+        return SummedUpdate(pick(self.row), pick(self.parts))
+
+    def total(self) -> torch.Tensor:
+        """fp32 ``[n, width]`` (diagnostics)."""
+        out = self.parts.float().sum(1) if self.parts is not None else 0.0
+        return out + self.row.float() if self.row is not None else out
+
+
 @torch.no_grad()
-def add_rmsnorm_shift(x_in, delta, weight, eps, *, x_out=None, shift=None, step=None, state=None):
-    """``s = x_in + delta`` (fp32 residual ``[n, width]``; ``delta`` in the storage dtype or ``None``), RMS norm with ``weight``,
+def add_rmsnorm_shift(x_in, delta, weight, eps, *, x_out=None, shift=None, step=None, state=None, out_scale: float = 1.0):
+    """``s = x_in + delta`` (fp32 residual ``[n, width]``; ``delta`` in the storage dtype, a :class:`SummedUpdate`, or ``None``),
+    RMS norm with ``weight``,
     and -- with ``shift`` -- the token shift ``h + (h_prev - h) * shift`` against the previous token's normed row of the same
     sequence (``step``: the ragged step's vectors; ``state``: fp32 ``[2, slots, width]`` of this layer run, the half named by the
-    sequence's parity is read, the other written).  Returns ``(y, residual)``: ``y`` in the storage dtype, ``residual`` the
+    sequence's parity is read, the other written).  ``y`` is multiplied by ``out_scale`` in fp32 before its one rounding.
+    Returns ``(y, residual)``: ``y`` in the storage dtype, ``residual`` the
     tensor that now holds ``s`` (``x_out``, or ``x_in`` when there is no ``delta``)."""
     L.require_cuda(x_in, weight)
     n, width = x_in.shape
     if x_in.dtype != torch.float32 or not x_in.is_contiguous():
         raise ValueError("add_rmsnorm_shift: the residual stream is contiguous fp32")
     dt = weight.dtype
-    if delta is not None:
-        if delta.dtype != dt or delta.shape != x_in.shape or not delta.is_contiguous():
+    parts = None
+    if isinstance(delta, SummedUpdate):
+        delta, parts = delta.row, delta.parts
+        if parts is not None and (parts.dtype != dt or parts.dim() != 3 or parts.shape[0] != n or parts.shape[2] != width
+                                  or not parts.is_contiguous() or not 1 <= parts.shape[1] <= 64):
+            raise ValueError("add_rmsnorm_shift: part rows are contiguous [n, 1..64, width] in the weights' dtype")
+    if delta is not None or parts is not None:
+        if delta is not None and (delta.dtype != dt or delta.shape != x_in.shape or not delta.is_contiguous()):
             raise ValueError("add_rmsnorm_shift: delta must match the residual's shape, in the weights' dtype")
         if x_out is None:
             x_out = torch.empty_like(x_in)
@@ -376,13 +407,46 @@ def add_rmsnorm_shift(x_in, delta, weight, eps, *, x_out=None, shift=None, step=
             raise ValueError("add_rmsnorm_shift: the token shift needs the step's vectors and an fp32 [2, slots, width] state")
         if step.num_tokens != n:
             raise ValueError("add_rmsnorm_shift: the step describes another number of tokens")
+    updated = delta is not None or parts is not None
     L.check(L.lib().ll_add_rmsnorm_shift(
-        x_in.data_ptr(), L.ptr(delta), L.ptr(x_out) if delta is not None else 0, weight.data_ptr(), L.ptr(shift), y.data_ptr(),
+        x_in.data_ptr(), L.ptr(delta), L.ptr(x_out) if updated else 0, weight.data_ptr(), L.ptr(shift), y.data_ptr(),
         n, width, float(eps), *( (step.tok_seq.data_ptr(), step.seq_start.data_ptr(), step.seq_first_pos.data_ptr(),
                                   step.seq_slot.data_ptr(), step.seq_parity.data_ptr(), state.data_ptr(), state.shape[1] * width)
                                  if shift is not None else (0, 0, 0, 0, 0, 0, 0) ),
-        L.dtype_code(dt), L.stream_ptr()), "add_rmsnorm_shift")
-    return y, (x_out if delta is not None else x_in)
+        L.ptr(parts), parts.shape[1] if parts is not None else 0, float(out_scale), L.dtype_code(dt), L.stream_ptr()),
+        "add_rmsnorm_shift")
+    return y, (x_out if updated else x_in)
+
+
+@torch.no_grad()
+def embed_pair(tokens: torch.Tensor, embed: torch.Tensor, scale: float = 1.0, pair: torch.Tensor | None = None,
+               mul_prev: int = 0, mul_cur: int = 0, step=None, state: torch.Tensor | None = None) -> torch.Tensor:
+    """The fp32 residual stream of a step's tokens: ``embed[token] * scale`` plus, with ``pair [buckets + 1, width]``, the row
+    ``(previous token * mul_prev + token * mul_cur) mod buckets`` of that table -- its last row for a sequence's first token.
+    The previous token of a run's first token is carried in ``state`` (int32 ``[2, slots]``: the half named by the sequence's
+    parity is read; the run's last token goes to the other half)."""
+    L.require_cuda(tokens, embed, pair, state)
+    if tokens.dtype != torch.int32:
+        tokens = tokens.to(torch.int32)
+    n, (vocab, width) = tokens.numel(), embed.shape
+    if not tokens.is_contiguous() or not embed.is_contiguous():
+        raise ValueError("embed_pair: contiguous token ids and table")
+    args = (0, 0, 0, 0, 0, 0, 0)
+    buckets = 0
+    if pair is not None:
+        if pair.dtype != embed.dtype or pair.dim() != 2 or pair.shape[1] != width or pair.shape[0] < 2 or not pair.is_contiguous():
+            raise ValueError("embed_pair: the pair table is [buckets + 1, width] in the embedding's dtype")
+        if step is None or state is None or state.dtype != torch.int32 or state.dim() != 2 or state.shape[0] != 2 \
+                or not state.is_contiguous() or step.num_tokens != n:
+            raise ValueError("embed_pair: the pair table needs the step's vectors and an int32 [2, slots] state")
+        buckets = pair.shape[0] - 1
+        args = (step.tok_seq.data_ptr(), step.seq_start.data_ptr(), step.seq_first_pos.data_ptr(), step.seq_slot.data_ptr(),
+                step.seq_parity.data_ptr(), state.data_ptr(), state.shape[1])
+    x = torch.empty(n, width, dtype=torch.float32, device=embed.device)
+    L.check(L.lib().ll_embed_pair(x.data_ptr(), tokens.data_ptr(), embed.data_ptr(), vocab, float(scale), L.ptr(pair), buckets,
+                                  int(mul_prev), int(mul_cur), n, width, *args, L.dtype_code(embed.dtype), L.stream_ptr()),
+            "embed_pair")
+    return x
 
 
 @torch.no_grad()
@@ -471,14 +535,17 @@ def gated_group_norm(x: torch.Tensor, update: "GatedUpdate | None", next_weight,
     return h
 
 
-_GLU_KINDS = {"silu": 0, "gelu_tanh": 1, "sigmoid": 2}
+_GLU_KINDS = {"silu": 0, "gelu_tanh": 1, "sigmoid": 2, "clamped": 3}
 
 
 @torch.no_grad()
-def glu_act(gate: torch.Tensor, ff: int, kind: str, up: torch.Tensor | None = None) -> torch.Tensor:
+def glu_act(gate: torch.Tensor, ff: int, kind: str, up: torch.Tensor | None = None, *, limit: float = 0.0, slope: float = 1.0,
+            out: torch.Tensor | None = None) -> torch.Tensor:
     """``act(gate[:, :ff]) * up[:, :ff]``; without ``up`` the rows of ``gate`` hold ``[gate | up]``.  Both may be wider,
-    row-strided views (column ranges of a fused projection).  ``kind``: ``"silu"``, ``"gelu_tanh"`` or ``"sigmoid"``.  fp32
-    arithmetic, one rounding to the storage dtype."""
+    row-strided views (column ranges of a fused projection).  ``kind``: ``"silu"``, ``"gelu_tanh"``, ``"sigmoid"``, or
+    ``"clamped"``: ``g sigmoid(slope g) (u + 1)`` with ``g = min(gate, limit)``, ``u = clamp(up, -limit, limit)``.  fp32
+    arithmetic, one rounding to the storage dtype.  ``out``: a ``[n, ff]`` view with a unit inner stride (a column range of the
+    next projection's input)."""
     if up is None:
         if gate.shape[1] < 2 * ff:
             raise ValueError("glu_act: rows hold [gate | up]")
@@ -487,9 +554,13 @@ def glu_act(gate: torch.Tensor, ff: int, kind: str, up: torch.Tensor | None = No
     if gate.dim() != 2 or up.dim() != 2 or gate.stride(1) != 1 or up.stride(1) != 1 or gate.shape[1] < ff or up.shape[1] < ff \
             or up.dtype != gate.dtype or up.shape[0] != gate.shape[0]:
         raise ValueError("glu_act: gate and up are [n, >= ff] of one dtype with unit inner strides")
-    out = torch.empty(gate.shape[0], ff, dtype=gate.dtype, device=gate.device)
-    L.check(L.lib().ll_glu_act(out.data_ptr(), gate.data_ptr(), gate.stride(0), up.data_ptr(), up.stride(0), gate.shape[0], int(ff),
-                               _GLU_KINDS[kind], L.dtype_code(gate.dtype), L.stream_ptr()), "glu_act")
+    if out is None:
+        out = torch.empty(gate.shape[0], ff, dtype=gate.dtype, device=gate.device)
+    elif out.dtype != gate.dtype or tuple(out.shape) != (gate.shape[0], ff) or out.stride(1) != 1 or not out.is_cuda:
+        raise ValueError("glu_act: out is [n, ff] in the inputs' dtype with a unit inner stride")
+    L.check(L.lib().ll_glu_act(out.data_ptr(), out.stride(0) if out.shape[0] > 1 else max(out.stride(0), ff), gate.data_ptr(),
+                               gate.stride(0), up.data_ptr(), up.stride(0), gate.shape[0], int(ff), _GLU_KINDS[kind], float(limit),
+                               float(slope), L.dtype_code(gate.dtype), L.stream_ptr()), "glu_act")
     return out
 
 

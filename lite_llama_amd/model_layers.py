@@ -16,13 +16,19 @@ description, out of mixers that take a ragged step (executor/ragged.py) and keep
   * :class:`GatedMLP`          ``down(act(gate h) * up h)`` (silu or tanh-gelu)
   * :class:`SparseMoE`         sigmoid router over expert groups, grouped expert products, a shared expert with a per-token
                                scale (kernels/fused_moe.py)
+  * :class:`ConvRotaryAttention`  biased q / k / v behind a short causal convolution over time, a rotation of entry pairs, unit
+                               RMS norm of q / k heads, a sliding window that also keeps a sequence's first keys, a sink of score
+                               0 in the denominator, values blended with those of the first such layer (kernels/attention.py)
+  * :class:`ChosenSoftmaxMoE`  the largest router logits choose the experts, their weights are the softmax over the chosen
+                               logits alone (kernels/fused_moe.py)
 
 The residual stream is fp32 throughout; every layer's residual add is fused into the norm that follows it
 (kernels/norm_act.py::add_rmsnorm_shift, which also applies the token shift in front of a mixer; or
 kernels/norm_act.py::gated_group_norm for layers that wrap each sublayer in two grouped norms and gate its result).
 Projections run through the framework's linear layers (library GEMM for unquantised weights), with everything that reads one
-input fused into one launch at load time.  Families: Rakevik (``"architecture": "Rakevik"``: :class:`MixerLayer`) and
-Rukedra (:class:`SandwichLayer`).
+input fused into one launch at load time.  Families: Rakevik (``"architecture": "Rakevik"``: :class:`MixerLayer`),
+Rukedra (:class:`SandwichLayer`) and Fekanex (:class:`ParallelLayer`: one norm per layer, mixer and feed-forward read its
+output side by side, and -- with a dense feed-forward -- share ONE input projection and ONE output projection).
 """
 
 from __future__ import annotations
@@ -38,9 +44,10 @@ import torch.nn.functional as F
 
 from .distributed.parallel_state import get_tp_world_size
 from .kernels.activations import xielu
-from .kernels.attention import latent_kv_prep, qk_norm_cache, ragged_attention, rotate_pairs
+from .kernels.attention import conv_rope_cache, latent_kv_prep, qk_norm_cache, ragged_attention, rotate_pairs
 from .kernels.fused_moe import group_router, sparse_glu_experts
-from .kernels.norm_act import GatedUpdate, add_rmsnorm_shift, cast_pair, gated_group_norm, glu_act, residual_set, softcap_
+from .kernels.norm_act import (GatedUpdate, SummedUpdate, add_rmsnorm_shift, cast_pair, embed_pair, gated_group_norm, glu_act,
+                               residual_set, softcap_)
 from .kernels.recurrent import gated_linear_scan, mingru_scan
 from .linear import ReplicatedLinear
 
@@ -88,7 +95,7 @@ class RotarySpec:
 
 @dataclass(frozen=True)
 class MixerSpec:
-    kind: str                   # "attention" | "hgrn2" | "latent_attention" | "mingru"
+    kind: str                   # "attention" | "hgrn2" | "latent_attention" | "mingru" | "conv_attention"
     heads: int = 1
     dim: int = 0                # per-head query / key width (latent attention: the unrotated part)
     vdim: int = 0               # per-head value width
@@ -99,7 +106,13 @@ class MixerSpec:
     rot_dim: int = 0            # latent attention: rotated query / key entries per head (the key's are shared by all heads)
     kv_rank: int = 0            # latent attention: width of the cached key/value latent
     q_rank: int = 0             # latent attention: width of the query latent (0: queries are projected directly)
-    window: int = 0             # latent attention: 0 = causal, else the last `window` positions are seen
+    window: int = 0             # latent / conv attention: 0 = causal, else the last `window` positions are seen
+    keep_first: int = 0         # conv attention: with a window, the sequence's first positions that stay visible
+    bias: bool = False          # conv attention: q / k / v projections carry a bias
+    conv_taps: int = 0          # conv attention: taps of the causal convolution over time behind the projections (0: none)
+    unit_norm: bool = False     # conv attention: q / k heads divided by their root mean square (no weight) after the rotation
+    unit_sink: bool = False     # conv attention: a key of score 0 without a value in every softmax denominator
+    value_mix: bool = False     # conv attention: values blended with those of the first layer that says so
     out_gate: bool = False      # latent attention: heads times sigmoid(W_g h) before the output projection
     rotary: RotarySpec | None = None
     width: int = 0              # mingru: channels of the recurrence
@@ -109,7 +122,9 @@ class MixerSpec:
 class MlpSpec:
     kind: str = "dense"         # "dense" | "moe"
     ff: int = 0                 # dense: hidden width; moe: hidden width of one expert
-    act: str = "xielu"          # dense: "xielu" (up / down) | "gelu_tanh" (gate / up / down)
+    act: str = "xielu"          # dense: "xielu" (up / down) | "gelu_tanh" | "clamped" (gate / up / down)
+    limit: float = 0.0          # "clamped": gate <= limit, |up| <= limit
+    scoring: str = "sigmoid"    # moe: "sigmoid" (scores over groups) | "softmax_chosen" (largest logits, softmax over them)
     experts: int = 0
     top: int = 0
     group_count: int = 1
@@ -141,6 +156,13 @@ class LayeredGeometry:
     sandwich: bool = False      # every sublayer between two norms, its result gated by sigmoid(W_r h + b_r)
     norm_groups: int = 1        # norms are taken over this many equal consecutive parts of the row
     logit_softcap: float = 0.0  # logits <- cap tanh(logits / cap)
+    parallel: bool = False      # one norm per layer; mixer and feed-forward both read it, their results are added together
+    embed_scale: float = 1.0    # input = embedding row times this
+    pair_buckets: int = 0       # > 0: plus row hash(previous token, token) of a [buckets + 1, width] table (last row: no previous)
+    pair_mul_prev: int = 0      # hash = (previous * mul_prev + token * mul_cur) mod buckets
+    pair_mul_cur: int = 0
+    logit_scale: float = 1.0    # logits = head(norm(x)) times this
+    tied_head: bool = False     # the output head is the embedding table
     extra: dict = field(default_factory=dict, compare=False)
 
     @property
@@ -161,6 +183,8 @@ class LayeredGeometry:
     def from_config(config: Mapping, name: str = "rakevik") -> "LayeredGeometry":
         if name == "rukedra":
             return _rukedra_geometry(config, name)
+        if name == "fekanex":
+            return _fekanex_geometry(config, name)
         layers = []
         for entry in config["layers"]:
             m, kind = entry["mixer"], entry["type"]
@@ -236,6 +260,48 @@ def _rukedra_geometry(config: Mapping, name: str) -> LayeredGeometry:
     return LayeredGeometry(name=name, vocab_size=int(config["vocab"]), width=int(config["width"]), eps=float(norm["eps"]),
                            layers=tuple(layers), token_shift=False, sandwich=True, norm_groups=groups,
                            logit_softcap=float(config.get("logit_softcap") or 0.0))
+
+
+def _fekanex_geometry(config: Mapping, name: str) -> LayeredGeometry:
+    """Fekanex: attention behind short convolutions with a rotation, unit q / k norms, a window that keeps the first keys and
+    a unit sink; dense (clamped GLU) or mixture-of-experts (softmax over the chosen logits) feed-forwards beside the mixer
+    under one norm; a hashed token-pair table added to the scaled embedding; logits from the embedding table, scaled."""
+    layers = []
+    for index, entry in enumerate(config["layers"]):
+        m, kind = entry["mixer"], entry["type"]
+        if kind != "attention":
+            raise ValueError(f"unsupported mixer type {kind!r}; supported: attention")
+        rot = RotarySpec.from_config(m["rot"]) if m.get("rot") else None
+        mask = m.get("mask") or {}
+        spec = MixerSpec("conv_attention", heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                         kv_heads=int(m.get("kv_heads") or m["heads"]), scale=float(m["scale"]), rotary=rot,
+                         window=int(mask.get("size") or 0), keep_first=int(mask.get("keep_first") or 0), bias=True,
+                         conv_taps=int(m.get("conv") or 0), unit_norm=True, unit_sink=True, value_mix=bool(m.get("v_mix")))
+        if spec.heads % spec.kv_heads:
+            raise ValueError(f"layer {index}: {spec.heads} query heads do not divide over {spec.kv_heads} key/value heads")
+        if rot is not None and (rot.dims > spec.dim or rot.dims % 2):
+            raise ValueError(f"layer {index}: {rot.dims} rotated entries do not fit heads of {spec.dim}")
+        mlp = entry.get("mlp")
+        if mlp is None:
+            mspec = None
+        elif mlp.get("kind", "dense") == "dense":
+            mspec = MlpSpec("dense", ff=int(mlp["ff"]), act="clamped", limit=float(mlp["limit"]))
+        elif mlp["kind"] == "moe":
+            r = mlp["router"]
+            mspec = MlpSpec("moe", ff=int(mlp["expert"]["ff"]), act="silu", experts=int(r["experts"]), top=int(r["top"]),
+                            scoring="softmax_chosen")
+            if not 1 <= mspec.top <= mspec.experts:
+                raise ValueError(f"layer {index}: {mspec.top} of {mspec.experts} experts cannot be chosen")
+        else:
+            raise ValueError(f"unsupported feed-forward kind {mlp.get('kind')!r}; supported: dense, moe")
+        layers.append(LayerSpec(spec, ff=mspec.ff if mspec else 0, mlp_kind=mspec.kind if mspec else "dense", mlp=mspec))
+    emb = config.get("embedding") or {}
+    pair = emb.get("bigram") or {}
+    return LayeredGeometry(name=name, vocab_size=int(config["vocab"]), width=int(config["width"]), eps=float(config["norm"]["eps"]),
+                           layers=tuple(layers), token_shift=False, parallel=True, embed_scale=float(emb.get("scale", 1.0)),
+                           pair_buckets=int(pair.get("buckets") or 0), pair_mul_prev=int(pair.get("mul_prev") or 0),
+                           pair_mul_cur=int(pair.get("mul_cur") or 0), logit_scale=float(config.get("logit_scale", 1.0)),
+                           tied_head=True)
 
 
 def _linear(inp: int, out: int) -> ReplicatedLinear:
@@ -466,7 +532,70 @@ class SparseMoE(nn.Module):
         return y, (rows[:, 2 * s.shared_ff:] if self.extra else None), shared, scale
 
 
-MIXERS = {"attention": SinkAttention, "hgrn2": GatedLinearMixer, "latent_attention": LatentAttention, "mingru": MinGRU}
+class ConvRotaryAttention(nn.Module):
+    """``q | k | v`` (and ``extra`` columns of the layer) in one projection; bias, convolution over time, rotation, unit q / k
+    norms, value blend and the cache write in one launch; attention over the paged cache with a window, kept first keys and a
+    sink of score 0.  The heads' outputs go to ``out`` (a column range of the layer's output projection input): the output
+    projection is the layer's."""
+
+    def __init__(self, width: int, spec: MixerSpec, eps: float, extra: int = 0):
+        super().__init__()
+        self.spec, self.eps, self.extra = spec, eps, extra
+        s = spec
+        self.channels = (s.heads + s.kv_heads) * s.dim + s.kv_heads * s.vdim
+        self.in_proj = _linear(width, self.channels + extra)
+        self.qkv_bias = _vector(self.channels) if s.bias else None
+        self.conv_weight = (nn.Parameter(torch.zeros(self.channels, s.conv_taps, dtype=torch.float16), requires_grad=False)
+                            if s.conv_taps else None)
+        self.value_blend = _vector(1) if s.value_mix else None
+        self._freq_values, self.amp = s.rotary.table() if s.rotary is not None else ([], 1.0)
+        self.pairs = len(self._freq_values)
+        self._freq = None   # fp32 on the device of the first step (not a buffer: a module-wide cast must not touch the angles)
+        self._sink = None   # zeros [heads]: exp(0) = 1 in every denominator
+
+    def cache_run(self) -> dict:
+        s = self.spec
+        return {"kind": "attention", "kv_heads": s.kv_heads, "dk": s.dim, "dv": s.vdim, "conv_taps": s.conv_taps,
+                "conv_channels": self.channels, "value_mix": s.value_mix}
+
+    def forward(self, h, step, cache, run: int, token_table, out=None):
+        s = self.spec
+        rows = self.in_proj(h)
+        k_cache, v_cache = cache.kv_buffer[run]
+        if self.pairs and (self._freq is None or self._freq.device != h.device):
+            self._freq = torch.tensor(self._freq_values, dtype=torch.float64).to(torch.float32).to(h.device)
+        if s.unit_sink and (self._sink is None or self._sink.device != h.device or self._sink.dtype != h.dtype):
+            self._sink = torch.zeros(s.heads, dtype=h.dtype, device=h.device)
+        source = cache.value_source[run]
+        q = conv_rope_cache(rows, s.heads, s.kv_heads, s.dim, s.vdim, step, k_cache, v_cache, bias=self.qkv_bias,
+                            conv_weight=self.conv_weight, conv_state=cache.conv[run], freq=self._freq, pairs=self.pairs,
+                            amp=self.amp, unit_norm=s.unit_norm, eps=self.eps,
+                            v_source=cache.kv_buffer[source][1] if source is not None else None,
+                            v_blend=self.value_blend if source is not None else None)
+        o = ragged_attention(q, k_cache, v_cache, s.scale, step, token_table, sink=self._sink if s.unit_sink else None,
+                             window=s.window, keep_first=s.keep_first, out=out)
+        return o, (rows[:, self.channels:] if self.extra else None)
+
+
+class ChosenSoftmaxMoE(nn.Module):
+    """The ``top`` largest router logits (fp32) choose a token's experts; their weights are the softmax over the chosen logits
+    alone.  Experts are gated feed-forwards without biases, run as grouped products over slots sorted by expert.  The slots'
+    rows are NOT summed here: they ride into the norm launch that follows."""
+
+    def __init__(self, width: int, spec: MlpSpec):
+        super().__init__()
+        self.spec = spec
+        self.router_weight = nn.Parameter(torch.zeros(spec.experts, width, dtype=torch.float16), requires_grad=False)
+        self.gate_up_weight = nn.Parameter(torch.zeros(spec.experts, 2 * spec.ff, width, dtype=torch.float16), requires_grad=False)
+        self.down_weight = nn.Parameter(torch.zeros(spec.experts, width, spec.ff, dtype=torch.float16), requires_grad=False)
+
+    def forward(self, h):
+        ids, weights, _ = group_router(h, self.router_weight, self.spec.top, scoring=self.spec.scoring)
+        return sparse_glu_experts(h, self.gate_up_weight, self.down_weight, ids, weights)
+
+
+MIXERS = {"attention": SinkAttention, "hgrn2": GatedLinearMixer, "latent_attention": LatentAttention, "mingru": MinGRU,
+          "conv_attention": ConvRotaryAttention}
 
 
 class MixerLayer(nn.Module):
@@ -520,6 +649,38 @@ class SandwichLayer(nn.Module):
         return x, pending
 
 
+class ParallelLayer(nn.Module):
+    """``x <- x + (mixer(h) + feed_forward(h))`` with ``h = norm(x)``: one norm, both sublayers read it.  With a dense
+    feed-forward, ``q | k | v | gate | up`` are ONE input projection and ``[heads' outputs | activation]`` go through ONE output
+    projection ``[W_o | W_down]``, whose fp32 accumulation is the sum of the two sublayers.  With experts, the mixer's output
+    projection gives one row and the experts' slots ride beside it as a :class:`SummedUpdate` into the next norm launch."""
+
+    slope = 1.702   # inside the sigmoid of the clamped GLU
+
+    def __init__(self, geo: LayeredGeometry, spec: LayerSpec):
+        super().__init__()
+        self.eps = geo.eps
+        w, m = geo.width, spec.mixer
+        self.norm1_weight = _vector(w)
+        self.dense = spec.mlp if (spec.mlp is not None and spec.mlp.kind == "dense") else None
+        ff = self.dense.ff if self.dense is not None else 0
+        self.mixer = MIXERS[m.kind](w, m, geo.eps, extra=2 * ff)
+        self.heads_width = m.heads * m.vdim
+        self.out_proj = _linear(self.heads_width + ff, w)
+        self.experts = ChosenSoftmaxMoE(w, spec.mlp) if (spec.mlp is not None and spec.mlp.kind == "moe") else None
+
+    def forward(self, x, pending, step, cache, run: int, token_table):
+        """``(x, pending)``: the fp32 residual (updated in place) and the update still to enter it.  Returns the same pair."""
+        h, x = add_rmsnorm_shift(x, pending, self.norm1_weight, self.eps, x_out=x)
+        ff = self.dense.ff if self.dense is not None else 0
+        mixed = torch.empty(h.shape[0], self.heads_width + ff, dtype=h.dtype, device=h.device)
+        _, gate_up = self.mixer(h, step, cache, run, token_table, out=mixed[:, :self.heads_width])
+        if ff:
+            glu_act(gate_up, ff, self.dense.act, limit=self.dense.limit, slope=self.slope, out=mixed[:, self.heads_width:])
+        row = self.out_proj(mixed)
+        return x, SummedUpdate(row, self.experts(h) if self.experts is not None else None)
+
+
 # ------------------------------------------------------------------------------------- #
 # the model
 # ------------------------------------------------------------------------------------- #
@@ -533,7 +694,7 @@ class LayeredLM(nn.Module):
         self.geo = geo
         self.embed_tokens = nn.Embedding(geo.vocab_size, geo.width, dtype=torch.float16)
         self.embed_tokens.weight.requires_grad_(False)
-        make = SandwichLayer if geo.sandwich else MixerLayer
+        make = SandwichLayer if geo.sandwich else ParallelLayer if geo.parallel else MixerLayer
         # a layer that borrows weights IS the other layer's module (which may come later in the stack); its cache run stays its own
         built = [make(geo, spec) if spec.weights_of is None else None for spec in geo.layers]
         self.layers = nn.ModuleList(built[i] if spec.weights_of is None else built[spec.weights_of] for i, spec in enumerate(geo.layers))
@@ -542,6 +703,11 @@ class LayeredLM(nn.Module):
             self.loop_step = nn.Parameter(torch.zeros(geo.loop_times, geo.width, dtype=torch.float16), requires_grad=False)
         self.norm_weight = _vector(geo.width)
         self.lm_head = _linear(geo.width, geo.vocab_size)
+        if geo.tied_head:   # (one parameter: it is listed, loaded and cast as the embedding table)
+            self.lm_head.weight = self.embed_tokens.weight
+        if geo.pair_buckets:
+            self.pair_table = nn.Parameter(torch.zeros(geo.pair_buckets + 1, geo.width, dtype=torch.float16), requires_grad=False)
+        self.needs_previous_token = geo.pair_buckets > 0
         self.run_order = geo.run_order()
         self.to(dtype)
 
@@ -565,7 +731,11 @@ class LayeredLM(nn.Module):
         """``token_ids [n]`` int64 of the step's flat token array.  ``logits_rows``: int64 indices into it (``None``: no
         logits, the step only fills cache and state).  ``collect_layers``: a list that receives the fp32 residual stream after
         every layer run (diagnostics; costs one add per run)."""
-        x0 = residual_set(F.embedding(token_ids, self.embed_tokens.weight))
+        if self.geo.pair_buckets or self.geo.embed_scale != 1.0:
+            x0 = embed_pair(token_ids, self.embed_tokens.weight, self.geo.embed_scale, self.pair_table if self.geo.pair_buckets else None,
+                            self.geo.pair_mul_prev, self.geo.pair_mul_cur, step, cache.prev_token)
+        else:
+            x0 = residual_set(F.embedding(token_ids, self.embed_tokens.weight))
         x, delta = (x0.clone() if self.geo.looped else x0), None  # (layers update the residual in place; x0 is read again)
         for run, (index, pass_no, first) in enumerate(self.run_order):
             if first:
@@ -577,6 +747,8 @@ class LayeredLM(nn.Module):
                     seen = x.clone()
                     gated_group_norm(seen, delta, None, self.geo.eps, self.geo.norm_groups)
                     collect_layers.append(seen)
+                elif isinstance(delta, SummedUpdate):
+                    collect_layers.append(x + delta.total())
                 else:
                     collect_layers.append(x + delta.float() if delta is not None else x.clone())
         if logits_rows is None:
@@ -586,8 +758,11 @@ class LayeredLM(nn.Module):
             h = gated_group_norm(x, delta.rows(logits_rows) if delta is not None else None, self.norm_weight, self.geo.eps,
                                  self.geo.norm_groups)
         else:
-            delta = delta[logits_rows].contiguous() if delta is not None else None
-            h, _ = add_rmsnorm_shift(x, delta, self.norm_weight, self.geo.eps, x_out=x)
+            if isinstance(delta, SummedUpdate):
+                delta = delta.rows(logits_rows)
+            else:
+                delta = delta[logits_rows].contiguous() if delta is not None else None
+            h, _ = add_rmsnorm_shift(x, delta, self.norm_weight, self.geo.eps, x_out=x, out_scale=self.geo.logit_scale)
         logits = self.lm_head(h)
         return softcap_(logits, self.geo.logit_softcap) if self.geo.logit_softcap else logits
 
@@ -611,15 +786,19 @@ class LayeredLM(nn.Module):
             leaf = name.rsplit(".", 1)[-1]
             if name.endswith("proj.weight") or name.endswith("lm_head.weight"):
                 fill(p, std=1.0 / (p.shape[1] ** 0.5))
-            elif name == "embed_tokens.weight":
+            elif name in ("embed_tokens.weight", "pair_table"):
                 fill(p, std=1.0)
             elif leaf in ("norm1_weight", "norm2_weight", "norm_weight", "q_norm_weight", "k_norm_weight", "out_norm_weight",
                           "norm1b_weight", "norm2b_weight", "kv_norm_weight"):
                 fill(p, std=0.1, mean=1.0)
             elif leaf in ("uk_weight", "uv_weight", "router_weight", "gate_up_weight", "down_weight", "shared_scale_weight"):
                 fill(p, std=1.0 / (p.shape[-1] ** 0.5))
-            elif leaf in ("rg1_bias", "rg2_bias", "z_bias", "x_bias"):
+            elif leaf in ("rg1_bias", "rg2_bias", "z_bias", "x_bias", "qkv_bias"):
                 fill(p, std=0.5)
+            elif leaf == "conv_weight":
+                fill(p, std=p.shape[1] ** -0.5)
+            elif leaf == "value_blend":
+                fill(p, lo=0.2, hi=0.6)
             elif leaf in ("shift", "lower"):
                 fill(p, lo=0.0, hi=0.9)
             elif leaf in ("f_bias", "sink", "act", "loop_step"):

@@ -42,10 +42,15 @@ class Region:
     part: int | None = None     # row block `part` of `parts` equal blocks (of the expert's slice if `expert` is set)
     parts: int = 2
     rows: tuple[int, int] | None = None   # (first row, count): one member of a projection fused from UNEQUAL members
+    cols: tuple[int, int] | None = None   # (first column, count): one member of a projection fused along its INPUT
 
     def __call__(self, param: torch.Tensor) -> torch.Tensor:
         view = param if self.expert is None else param[self.expert]
+        if self.cols is not None:
+            return view.narrow(1, self.cols[0], self.cols[1])
         if self.rows is not None:
+            if view.dim() == 1 and self.rows[1] == 1 and view.numel() > self.rows[0]:
+                return view[self.rows[0]]   # (a scalar tensor of the checkpoint fills one entry)
             return view.narrow(0, self.rows[0], self.rows[1])
         if self.part is not None:
             rows = view.shape[0] // self.parts
@@ -648,18 +653,72 @@ def _rukedra_translator(geo) -> Translator:
     return translate
 
 
+def _fekanex_translator(geo) -> Translator:
+    """Tensor names of a Fekanex checkpoint -> parameters of :class:`lite_llama_amd.model_layers.LayeredLM` built from
+    :class:`ParallelLayer`: ``mix.q / k / v`` (and, with a dense feed-forward, ``mlp.gate / up``) land in their row ranges of the
+    layer's one input projection, their biases and convolution taps in the same ranges of one bias vector and one tap matrix;
+    ``mix.o`` (and ``mlp.down``) in their COLUMN ranges of the one output projection; experts ``mlp.e<k>.*`` in the stacked
+    expert tensors.  The output head is the embedding table (no tensor of its own)."""
+    fixed = {"embed": "embed_tokens.weight", "bigram": "pair_table", "final.norm": "norm_weight"}
+    plain = {"norm1": "norm1_weight", "mlp.router": "experts.router_weight"}
+    expert_leaf = re.compile(r"^mlp\.e(\d+)\.(gate|up|down)$")
+
+    def fused(spec):
+        """``{checkpoint leaf: (parameter, Region)}`` of one layer."""
+        m, out = spec.mixer, {}
+        q, k, v = m.heads * m.dim, m.kv_heads * m.dim, m.kv_heads * m.vdim
+        for leaf, first, count in (("mix.q", 0, q), ("mix.k", q, k), ("mix.v", q + k, v)):
+            out[leaf] = ("mixer.in_proj.weight", Region(rows=(first, count)))
+            out[leaf + ".b"] = ("mixer.qkv_bias", Region(rows=(first, count)))
+            out[leaf + ".conv"] = ("mixer.conv_weight", Region(rows=(first, count)))
+        out["mix.vmix"] = ("mixer.value_blend", Region(rows=(0, 1)))
+        heads_width = m.heads * m.vdim
+        out["mix.o"] = ("out_proj.weight", Region(cols=(0, heads_width)))
+        if spec.mlp is not None and spec.mlp.kind == "dense":
+            ff = spec.mlp.ff
+            out["mlp.gate"] = ("mixer.in_proj.weight", Region(rows=(q + k + v, ff)))
+            out["mlp.up"] = ("mixer.in_proj.weight", Region(rows=(q + k + v + ff, ff)))
+            out["mlp.down"] = ("out_proj.weight", Region(cols=(heads_width, ff)))
+        return out
+
+    members = [fused(spec) for spec in geo.layers]
+
+    def translate(key: str) -> Target:
+        if key in fixed:
+            return fixed[key], whole
+        m = re.match(r"^l(\d+)\.(.+)$", key)
+        if m is None or int(m.group(1)) >= len(geo.layers):
+            return key, whole  # unknown: load_weights reports it
+        index, leaf = int(m.group(1)), m.group(2)
+        if leaf == "mix.vmix" and not geo.layers[index].mixer.value_mix:
+            return None  # (a blend weight of a layer that does not blend)
+        if leaf in members[index]:
+            name, region = members[index][leaf]
+            return f"layers.{index}.{name}", region
+        e = expert_leaf.match(leaf)
+        if e is not None:
+            k, proj = int(e.group(1)), e.group(2)
+            if proj == "down":
+                return f"layers.{index}.experts.down_weight", expert(k)
+            return f"layers.{index}.experts.gate_up_weight", expert_half(k, 0 if proj == "gate" else 1)
+        return f"layers.{index}.{plain.get(leaf, leaf)}", whole
+
+    return translate
+
+
 def _load_layered(config: Mapping, checkpoints_dir, device, dtype=None, **_):
     from .model_layers import LayeredGeometry, LayeredLM
 
     geo = LayeredGeometry.from_config(config, name=model_family(config))
     model = LayeredLM(geo, dtype=dtype or torch.bfloat16).to(device)
-    translator = _rukedra_translator(geo) if geo.sandwich else _layered_translator(geo)
+    translator = (_rukedra_translator(geo) if geo.sandwich else _fekanex_translator(geo) if geo.parallel
+                  else _layered_translator(geo))
     with torch.no_grad():
         load_weights(model, hf_weights_iterator(checkpoints_dir, device), translator)
     return model.eval()
 
 
-MODEL_FAMILIES: dict[str, Callable] = {"rakevik": _load_layered, "rukedra": _load_layered}
+MODEL_FAMILIES: dict[str, Callable] = {"rakevik": _load_layered, "rukedra": _load_layered, "fekanex": _load_layered}
 
 
 def load_pretrained(checkpoints_dir: str | Path, *, device: str | torch.device = "cuda", quantization: str | None = None,
