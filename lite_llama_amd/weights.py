@@ -43,14 +43,15 @@ class Region:
     parts: int = 2
     rows: tuple[int, int] | None = None   # (first row, count): one member of a projection fused from UNEQUAL members
     cols: tuple[int, int] | None = None   # (first column, count): one member of a projection fused along its INPUT
+    entry: int | None = None    # one entry of a vector, filled by a checkpoint tensor without dimensions
 
     def __call__(self, param: torch.Tensor) -> torch.Tensor:
         view = param if self.expert is None else param[self.expert]
         if self.cols is not None:
             return view.narrow(1, self.cols[0], self.cols[1])
+        if self.entry is not None:
+            return view[self.entry]
         if self.rows is not None:
-            if view.dim() == 1 and self.rows[1] == 1 and view.numel() > self.rows[0]:
-                return view[self.rows[0]]   # (a scalar tensor of the checkpoint fills one entry)
             return view.narrow(0, self.rows[0], self.rows[1])
         if self.part is not None:
             rows = view.shape[0] // self.parts
@@ -671,7 +672,7 @@ def _fekanex_translator(geo) -> Translator:
             out[leaf] = ("mixer.in_proj.weight", Region(rows=(first, count)))
             out[leaf + ".b"] = ("mixer.qkv_bias", Region(rows=(first, count)))
             out[leaf + ".conv"] = ("mixer.conv_weight", Region(rows=(first, count)))
-        out["mix.vmix"] = ("mixer.value_blend", Region(rows=(0, 1)))
+        out["mix.vmix"] = ("mixer.value_blend", Region(entry=0))
         heads_width = m.heads * m.vdim
         out["mix.o"] = ("out_proj.weight", Region(cols=(0, heads_width)))
         if spec.mlp is not None and spec.mlp.kind == "dense":
