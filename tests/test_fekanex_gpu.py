@@ -125,7 +125,8 @@ def test_router_chooses_the_largest_logits_and_weighs_them_by_their_own_softmax(
     want_ids, want_w = O.route(d(h), d(wr), top)
     assert extra is None and ids.dtype == torch.int32 and weights.dtype == torch.float32
     logits = d(h) @ d(wr).T
-    gap = (torch.topk(logits, min(top + 1, experts), -1).values.diff(dim=-1).abs().min(-1).values > 1e-4)   # (no close calls)
+    best = torch.topk(logits, min(top + 1, experts), -1).values
+    gap = best.diff(dim=-1).abs().min(-1).values > 1e-4 if best.shape[1] > 1 else torch.ones(n, dtype=torch.bool)   # (no close calls)
     assert gap.sum() > n // 2
     assert torch.equal(ids.cpu().long()[gap], want_ids[gap])
     _close(weights[gap.to(DEV)], want_w[gap], 1e-5)
@@ -147,7 +148,7 @@ def _conv_case(dtype, heads, kv_heads, dk, dv, taps, pairs, plan, lens, blend, u
     b = (torch.randn(channels) * 0.5).to(dtype) if bias else None
     cw = (torch.randn(channels, taps) * 0.6 + 0.3).to(dtype) if taps else None
     lam = torch.tensor([0.375]).to(dtype)
-    total_rows = sum(lens.values()) + 16
+    total_rows = 4 * max(lens.values()) + 16
     table = torch.randperm(total_rows)[:4 * max(lens.values())].view(4, -1).to(torch.int32)
     src = torch.randn(total_rows, kv_heads, dv).to(dtype)
     want = {}
@@ -338,9 +339,9 @@ def test_sink_of_score_zero_takes_the_weight_when_every_score_is_low(dtype, shap
     total = 300
     plan = [[(1, 0, 280)]] + [[(1, 280 + i, 1)] for i in range(20)]
     got, want = _attention_case(dtype, *shape, total, plan, 30, 2, low=True)
-    assert want.abs().max() < 1e-3 and got.float().abs().max() < 1e-3
+    assert want.abs().max() < 0.02 and (got.float().cpu() - want).abs().max() < 1e-3
     plain, _ = _attention_case(dtype, *shape, total, plan, 30, 2, low=True, sink=False)
-    assert plain.float().abs().max() > 0.05
+    assert plain.float().abs().max() > 0.5
     got, want = _attention_case(dtype, *shape, total, plan, 30, 2, scale=0.1)
     _close(got, want, 5e-5 if dtype == torch.float32 else 3e-2)
     none, _ = _attention_case(dtype, *shape, total, plan, 30, 2, scale=0.1, sink=False)
