@@ -99,6 +99,13 @@ def parse():
                     help="instead of the headline: prefill / decode throughput and per-kernel roofline fractions of the Rukedra "
                          "design (latent attention, minGRU, gated grouped norms, routed experts) at two model sizes beside the "
                          "closest llama-shaped model (benchmarks/rukedra_bench.py); --layered-dtype picks the dtype")
+    ap.add_argument("--fekanex", action="store_true",
+                    help="instead of the headline: prefill / decode throughput and per-kernel roofline fractions of the Fekanex "
+                         "design (convolved rotary attention with a window, kept first keys and a unit sink; clamped-GLU / expert "
+                         "feed-forwards beside the mixer) beside the closest llama-shaped model (benchmarks/fekanex_bench.py); "
+                         "--layered-dtype picks the dtype")
+    ap.add_argument("--fekanex-sizes", default="compact,wide", help="which size points of benchmarks/fekanex_bench.py::SIZES to run")
+    ap.add_argument("--fekanex-model-only", action="store_true", help="skip the per-kernel table (a short run for a kernel trace)")
     ap.add_argument("--rukedra-sizes", default="compact,wide", help="which size points of benchmarks/rukedra_bench.py::SIZES to run")
     ap.add_argument("--rukedra-model-only", action="store_true", help="skip the per-kernel table (a short run for a kernel trace)")
     ap.add_argument("--no-reference-order", action="store_true",
@@ -934,6 +941,11 @@ def main():
         from benchmarks.rukedra_bench import run as rukedra_run
 
         print(json.dumps(rukedra_run(args.layered_dtype, sizes=tuple(args.rukedra_sizes.split(",")), kernels=not args.rukedra_model_only)))
+        return
+    if args.fekanex:
+        from benchmarks.fekanex_bench import run as fekanex_run
+
+        print(json.dumps(fekanex_run(args.layered_dtype, sizes=tuple(args.fekanex_sizes.split(",")), kernels=not args.fekanex_model_only)))
         return
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         raise SystemExit(self_launch(args))

@@ -193,7 +193,187 @@ __device__ __forceinline__ float row16_sum(float v) {
   return v;
 }
 
-// 16-byte form of the kernel above: one 16-lane row per (token, item), lane r of the row owns the 16-byte pieces r, r + 16, ..
+// 16-byte form of the kernel above.  A workgroup owns 16 CONSECUTIVE TOKENS -- one per 16-lane row -- and a few items, which
+// its rows take in step: the tap weights and the bias of an item are fetched once for the sixteen tokens, and the rows a tap
+// reads are the neighbouring rows' own.  Lane r of a row owns the 16-byte pieces r, r + 16, .. of the head (up to four: widths
+// <= 512 sixteen-bit / 256 fp32 channels, multiples of 8 / 4; how many is a template constant, as are the taps (0 .. 4), so a
+// piece's tap weights sit in registers.  A token's cos / sin are computed once per workgroup, into LDS [16][2][pairs].  The same sums in
+// the same order as the plain form.
+template <int DT, int TAPS, int NPC>   // NPC: 16-byte pieces per lane (1, 2 or 4)
+__global__ __launch_bounds__(256) void conv_rope_cache_vec_kernel(
+    const void* __restrict__ qkv, int64_t ld, const void* __restrict__ bias, const void* __restrict__ conv_w,
+    void* __restrict__ conv_state, int64_t state_half, const float* __restrict__ freq, int pairs, float amp, int unit_norm,
+    float eps, const void* __restrict__ v_src, int64_t v_src_stride, const void* __restrict__ v_lam,
+    const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ select,
+    const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_first_pos, const int32_t* __restrict__ seq_slot,
+    const int32_t* __restrict__ seq_parity, void* __restrict__ q_out, void* __restrict__ k_cache, void* __restrict__ v_cache,
+    int64_t n, int heads, int kv_heads, int dk, int dv, int items_per_wg) {
+  constexpr int EPC = DT == LL_F32 ? 4 : 8;  // elements per 16-byte piece
+  typedef typename std::conditional<DT == LL_F32, float, uint16_t>::type elem;
+  struct alignas(16) Piece { elem e[EPC]; };
+  constexpr int BACK = TAPS > 1 ? TAPS - 1 : 0;
+  constexpr int WN = TAPS > 0 ? TAPS : 1;
+  extern __shared__ float rot_cs[];   // [16 tokens][cos | sin][pairs], times amp
+  const int items = heads + 2 * kv_heads;
+  const int trow = threadIdx.x >> 4, r = threadIdx.x & 15;
+  const int64_t t = (int64_t)blockIdx.x * 16 + trow;
+  if (t >= n) return;   // (whole 16-lane rows leave; nothing below synchronises across rows)
+  const int64_t channels = (int64_t)(heads + kv_heads) * dk + (int64_t)kv_heads * dv;
+  const int b = tok_seq[t];
+  const int pos = tok_pos[t], first = seq_first_pos[b];
+  const int in_run = pos - first;
+  const int item_lo = blockIdx.y * items_per_wg;
+  const int item_hi = item_lo + items_per_wg < items ? item_lo + items_per_wg : items;
+  float* my_cs = rot_cs + (int64_t)trow * 2 * pairs;
+  for (int i = r; i < pairs; i += 16) {
+    float sn, cs;
+    sincosf((float)pos * freq[i], &sn, &cs);
+    my_cs[i] = cs * amp;
+    my_cs[pairs + i] = sn * amp;
+  }
+  __builtin_amdgcn_wave_barrier();   // (written and read by the lanes of one row, which share a wave)
+  const bool last_of_run = t == seq_start[b + 1] - 1;
+  float lam = 0.f;
+  if (v_src) lam = ldv<DT>(v_lam, 0);
+  const int64_t crow = select[t];
+  const elem* rows = (const elem*)qkv;
+  const elem* old_state = rows;   // (never read without carried rows)
+  if constexpr (BACK > 0) old_state = (const elem*)conv_state + (int64_t)seq_parity[b] * state_half + (int64_t)seq_slot[b] * BACK * channels;
+  for (int item = item_lo; item < item_hi; ++item) {
+    const bool is_q = item < heads, is_v = item >= heads + kv_heads;
+    const int width = is_v ? dv : dk;
+    const int64_t col0 = is_v ? (int64_t)(heads + kv_heads) * dk + (int64_t)(item - heads - kv_heads) * dv : (int64_t)item * dk;
+    const int pieces = width / EPC;
+    float val[NPC][EPC];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < NPC; ++j) {
+      const int pc = r + 16 * j;
+      if (pc < pieces) {
+        const int64_t c = col0 + (int64_t)pc * EPC;
+        float bv[EPC], acc[EPC];
+#pragma unroll
+        for (int e = 0; e < EPC; ++e) bv[e] = acc[e] = 0.f;
+        // every load of the piece is issued before the first sum: the bias, the taps' rows (this step's, or the carried ones;
+        // a tap in front of position 0 re-reads the token's own row and counts as zero) and the EPC * TAPS contiguous tap
+        // weights of these channels (channel e, tap j at e * TAPS + j)
+        Piece braw, raw[WN], wraw[WN];
+        if (bias) braw = *reinterpret_cast<const Piece*>((const elem*)bias + c);
+#pragma unroll
+        for (int jt = 0; jt < WN; ++jt) {
+          const int dist = WN - 1 - jt;
+          const elem* src = rows + t * ld + c;
+          if constexpr (BACK > 0) {
+            if (dist <= pos && dist > in_run) src = old_state + (int64_t)(dist - in_run - 1) * channels + c;
+            else if (dist <= pos) src = rows + (t - dist) * ld + c;
+          }
+          raw[jt] = *reinterpret_cast<const Piece*>(src);
+          if constexpr (TAPS > 0) wraw[jt] = *reinterpret_cast<const Piece*>((const elem*)conv_w + c * TAPS + jt * EPC);
+        }
+        if (bias) {
+#pragma unroll
+          for (int e = 0; e < EPC; ++e) {
+            if constexpr (DT == LL_F32) bv[e] = braw.e[e];
+            else bv[e] = to_f32<DT>(braw.e[e]);
+          }
+        }
+        float w[WN][EPC];
+        if constexpr (TAPS > 0) {
+#pragma unroll
+          for (int k = 0; k < TAPS; ++k) {
+#pragma unroll
+            for (int e = 0; e < EPC; ++e) {
+              if constexpr (DT == LL_F32) w[k][e] = wraw[k].e[e];
+              else w[k][e] = to_f32<DT>(wraw[k].e[e]);
+            }
+          }
+        }
+#pragma unroll
+        for (int jt = 0; jt < WN; ++jt) {
+          const bool seen = WN - 1 - jt <= pos;
+#pragma unroll
+          for (int e = 0; e < EPC; ++e) {
+            float u;
+            if constexpr (DT == LL_F32) u = raw[jt].e[e];
+            else u = to_f32<DT>(raw[jt].e[e]);
+            if (bias) u += bv[e];
+            if constexpr (TAPS > 0) {
+              const int flat = e * TAPS + jt;
+              acc[e] += w[flat / EPC][flat % EPC] * (seen ? u : 0.f);
+            } else {
+              acc[e] = u;
+            }
+          }
+        }
+        if (!is_v) {
+#pragma unroll
+          for (int m = 0; m < EPC / 2; ++m) {
+            const int pi = pc * (EPC / 2) + m;
+            if (pi < pairs) {
+              const float cs = my_cs[pi], sn = my_cs[pairs + pi];
+              const float x0 = acc[2 * m], x1 = acc[2 * m + 1];
+              acc[2 * m] = x0 * cs - x1 * sn;
+              acc[2 * m + 1] = x1 * cs + x0 * sn;
+            }
+          }
+        }
+#pragma unroll
+        for (int e = 0; e < EPC; ++e) {
+          val[j][e] = acc[e];
+          ss += acc[e] * acc[e];
+        }
+      }
+    }
+    float mul = 1.0f;
+    if (!is_v && unit_norm) {
+      ss = row16_sum(ss);
+      mul = 1.0f / sqrtf(ss / (float)dk + eps);
+    }
+    const bool blend = is_v && v_src != nullptr;
+    elem* dst = is_q ? (elem*)q_out + (t * heads + item) * dk
+                     : is_v ? (elem*)v_cache + (crow * kv_heads + (item - heads - kv_heads)) * dv
+                            : (elem*)k_cache + (crow * kv_heads + (item - heads)) * dk;
+#pragma unroll
+    for (int j = 0; j < NPC; ++j) {
+      const int pc = r + 16 * j;
+      if (pc < pieces) {
+        Piece sraw;
+        if (blend) sraw = *reinterpret_cast<const Piece*>((const elem*)v_src + crow * v_src_stride + (int64_t)(item - heads - kv_heads) * dv + pc * EPC);
+        Piece o;
+#pragma unroll
+        for (int e = 0; e < EPC; ++e) {
+          float y = val[j][e] * mul;
+          if (blend) {
+            float sv;
+            if constexpr (DT == LL_F32) sv = sraw.e[e];
+            else sv = to_f32<DT>(sraw.e[e]);
+            y = (1.0f - lam) * y + lam * sv;
+          }
+          if constexpr (DT == LL_F32) o.e[e] = y;
+          else o.e[e] = from_f32<DT>(y);
+        }
+        *reinterpret_cast<Piece*>(dst + pc * EPC) = o;
+      }
+    }
+    if constexpr (BACK > 0) if (last_of_run) {   // the run's last token leaves the raw rows of the sequence's last TAPS - 1 positions
+      elem* new_state = (elem*)conv_state + (int64_t)(1 - seq_parity[b]) * state_half + (int64_t)seq_slot[b] * BACK * channels;
+#pragma unroll
+      for (int dist = 0; dist < BACK; ++dist) {             // state row `dist` = the position `dist` in front of this token
+        for (int pc = r; pc < pieces; pc += 16) {
+          const int64_t c = col0 + (int64_t)pc * EPC;
+          Piece v;
+#pragma unroll
+          for (int e = 0; e < EPC; ++e) v.e[e] = 0;
+          if (dist <= in_run) v = *reinterpret_cast<const Piece*>(rows + (t - dist) * ld + c);
+          else if (dist <= pos) v = *reinterpret_cast<const Piece*>(old_state + (int64_t)(dist - in_run - 1) * channels + c);
+          *reinterpret_cast<Piece*>(new_state + (int64_t)dist * channels + c) = v;
+        }
+      }
+    }
+  }
+}
+
+// 16-byte form of qk_norm_cache_kernel: one 16-lane row per (token, item), lane r of the row owns the 16-byte pieces r, r + 16, ..
 // of the head (up to four: widths <= 512 sixteen-bit / 256 fp32 channels, multiples of 8 / 4).
 template <int DT>
 __global__ __launch_bounds__(256) void qk_norm_cache_vec_kernel(
@@ -426,6 +606,37 @@ extern "C" int ll_conv_rope_cache(const void* qkv, int64_t ld, const void* bias,
   qkv, ld, bias, conv_w, (int)taps, conv_state, state_half, freq, (int)pairs, amp, unit_norm, eps, v_src, v_src_stride, v_lam, tok_seq, \
       tok_pos, select, seq_start, seq_first_pos, seq_slot, seq_parity, q_out, k_cache, v_cache, n, (int)heads, (int)kv_heads, (int)dk, \
       (int)dv
+  const int epc = dtype == LL_F32 ? 4 : 8;
+  const bool vec = taps <= 4 && dk % epc == 0 && dv % epc == 0 && ld % epc == 0 && widest <= 64 * epc && ll_aligned16(qkv) &&
+                   ll_aligned16(q_out) && ll_aligned16(k_cache) && ll_aligned16(v_cache) && (!bias || ll_aligned16(bias)) &&
+                   (!conv_w || ll_aligned16(conv_w)) && (taps <= 1 || ll_aligned16(conv_state)) &&
+                   (!v_src || (ll_aligned16(v_src) && v_src_stride % epc == 0));
+  if (vec) {
+    // 16 tokens per workgroup; the items of a token in groups of 4 when that still fills the chip, else one item each
+    const int64_t tiles = (n + 15) / 16, items = heads + 2 * kv_heads;
+    const int ipw = tiles * ((items + 3) / 4) >= 1024 ? 4 : 1;
+    const dim3 grid_v((unsigned)tiles, (unsigned)((items + ipw - 1) / ipw));
+    const size_t lds_v = sizeof(float) * 16 * 2 * (size_t)(pairs > 0 ? pairs : 1);
+#define LL_CRV_ARGS                                                                                                              \
+  qkv, ld, bias, conv_w, conv_state, state_half, freq, (int)pairs, amp, unit_norm, eps, v_src, v_src_stride, v_lam, tok_seq, tok_pos, \
+      select, seq_start, seq_first_pos, seq_slot, seq_parity, q_out, k_cache, v_cache, n, (int)heads, (int)kv_heads, (int)dk, (int)dv, ipw
+    const int npc = widest <= 16 * epc ? 1 : widest <= 32 * epc ? 2 : 4;
+#define CALL_N(DT, T)                                                                                            \
+  if (npc == 1) conv_rope_cache_vec_kernel<DT, T, 1><<<grid_v, 256, lds_v, st>>>(LL_CRV_ARGS);                   \
+  else if (npc == 2) conv_rope_cache_vec_kernel<DT, T, 2><<<grid_v, 256, lds_v, st>>>(LL_CRV_ARGS);              \
+  else conv_rope_cache_vec_kernel<DT, T, 4><<<grid_v, 256, lds_v, st>>>(LL_CRV_ARGS)
+#define CALL(DT)                              \
+  if (taps == 0) { CALL_N(DT, 0); }           \
+  else if (taps == 1) { CALL_N(DT, 1); }      \
+  else if (taps == 2) { CALL_N(DT, 2); }      \
+  else if (taps == 3) { CALL_N(DT, 3); }      \
+  else { CALL_N(DT, 4); }
+    LL_BY_DTYPE(dtype, CALL);
+#undef CALL
+#undef CALL_N
+#undef LL_CRV_ARGS
+    return LL_LAUNCH_CHECK();
+  }
 #define CALL(DT)                                                                               \
   if (widest <= 128) conv_rope_cache_kernel<DT, 1><<<grid, 256, 0, st>>>(LL_CR_ARGS);          \
   else if (widest <= 256) conv_rope_cache_kernel<DT, 2><<<grid, 256, 0, st>>>(LL_CR_ARGS);     \
