@@ -617,11 +617,16 @@ int ll_ragged_attention(const void* q, const void* k_cache, const void* v_cache,
  * y_t = sum_j conv_w[c][j] u_(t - taps + 1 + j) over the sequence's positions (zeros in front of position 0; taps == 0: none),
  * the raw rows of a sequence's last taps - 1 positions carried in conv_state [2][state_half] (half seq_parity read, the other
  * written; a slot is [taps - 1][channels], row d - 1 = position length - d); pairs (2i, 2i + 1), i < pairs, of every q / k head
- * rotated by pos * freq[i] with cos / sin times amp; q / k heads divided by sqrt(mean + eps) when unit_norm; v = (1 - lam) v +
+ * rotated by pos * freq[i] with cos / sin times amp (rot_table, when given, holds exactly these per token: ll_rotation_table;
+ * the 16-byte form needs it); q / k heads divided by sqrt(mean + eps) when unit_norm; v = (1 - lam) v +
  * lam v_src[select[t]] when v_src (rows of stride v_src_stride; lam = *v_lam) is given.  q -> q_out [n, heads, dk]; k, v ->
  * cache rows select[t]. */
+/* out [n][2 * pairs4] (fp32), pairs4 = pairs rounded up to a multiple of 4: entry pair i of token t at [t][2 i] =
+ * (cos(tok_pos[t] * freq[i]) * amp, sin(tok_pos[t] * freq[i]) * amp); the padding is not written. */
+int ll_rotation_table(const int32_t* tok_pos, const float* freq, int64_t pairs, float amp, float* out, int64_t n, void* stream);
 int ll_conv_rope_cache(const void* qkv, int64_t ld, const void* bias, const void* conv_w, int64_t taps, void* conv_state,
-                       int64_t state_half, const float* freq, int64_t pairs, float amp, int unit_norm, float eps,
+                       int64_t state_half, const float* freq, int64_t pairs, float amp, const float* rot_table,
+                       int unit_norm, float eps,
                        const void* v_src, int64_t v_src_stride, const void* v_lam, const int32_t* tok_seq,
                        const int32_t* tok_pos, const int32_t* select, const int32_t* seq_start, const int32_t* seq_first_pos,
                        const int32_t* seq_slot, const int32_t* seq_parity, void* q_out, void* k_cache, void* v_cache,

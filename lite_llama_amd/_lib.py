@@ -119,7 +119,8 @@ SIGNATURES = {
     "ll_gated_linear_scan": [P, P, P, L, P, P, P, F, P, L, L, L, L, P, P, P, P, L, L, P, I, P],
     "ll_qk_norm_cache": [P, L, P, P, F, F, L, P, P, P, P, P, L, L, L, L, L, I, P],
     "ll_ragged_attention": [P, P, P, P, L, P, P, P, P, F, P, L, L, L, L, L, L, L, L, L, L, I, P],
-    "ll_conv_rope_cache": [P, L, P, P, L, P, L, P, L, F, I, F, P, L, P, P, P, P, P, P, P, P, P, P, P, L, L, L, L, L, I, P],
+    "ll_rotation_table": [P, P, L, F, P, L, P],
+    "ll_conv_rope_cache": [P, L, P, P, L, P, L, P, L, F, P, I, F, P, L, P, P, P, P, P, P, P, P, P, P, P, L, L, L, L, L, I, P],
     "ll_ragged_attention_mfma_supported": [L, L, I],
     "ll_ragged_attention_partition": [],
     "ll_ragged_attention_mfma": [P, P, P, P, L, P, P, P, P, F, P, L, L, L, L, I, P, L, L, L, L, L, L, L, L, L, I, P],

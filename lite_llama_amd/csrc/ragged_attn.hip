@@ -8,6 +8,8 @@
 //                        taps - 1 projected rows of a sequence are carried in a state slot), rotation of entry pairs of q / k
 //                        heads, unit RMS norm of q / k heads, values blended with the values another layer cached for the same
 //                        token; queries out, keys and values into the cache rows of their tokens
+//   ll_rotation_table    cos / sin (times an amplitude) of position * frequency per token and entry pair, once per step for all
+//                        layers and heads that rotate alike
 //   ll_ragged_attention  every token of the step against keys 0 .. its own position of its sequence, read through the
 //                        per-token row table; scores, softmax and the running output in fp32; optionally only the last
 //                        `window` keys plus the sequence's first `keep_first`
@@ -72,6 +74,9 @@ __global__ __launch_bounds__(256) void qk_norm_cache_kernel(
   }
 }
 
+// floats per token of a rotation table: (cos, sin) per pair, the pairs padded to a multiple of four (32-byte pieces stay inside)
+__host__ __device__ __forceinline__ int64_t rot_stride(int64_t pairs) { return 2 * ((pairs + 3) & ~(int64_t)3); }
+
 // One wave per (token, item): items 0 .. H - 1 = query heads, H .. H + G - 1 = key heads, then G value heads.  Lane l owns the
 // entry pairs l, l + 64, .. of its head (NP of them).  Per channel, in fp32:
 //   u_p   = projected row of position p (+ bias): this step's rows, or -- in front of the run -- the sequence's state slot, which
@@ -85,7 +90,8 @@ __global__ __launch_bounds__(256) void qk_norm_cache_kernel(
 template <int DT, int NP>
 __global__ __launch_bounds__(256) void conv_rope_cache_kernel(
     const void* __restrict__ qkv, int64_t ld, const void* __restrict__ bias, const void* __restrict__ conv_w, int taps,
-    void* __restrict__ conv_state, int64_t state_half, const float* __restrict__ freq, int pairs, float amp, int unit_norm,
+    void* __restrict__ conv_state, int64_t state_half, const float* __restrict__ freq, int pairs, float amp,
+    const float* __restrict__ rot_table, int unit_norm,
     float eps, const void* __restrict__ v_src, int64_t v_src_stride, const void* __restrict__ v_lam,
     const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ select,
     const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_first_pos, const int32_t* __restrict__ seq_slot,
@@ -133,8 +139,15 @@ __global__ __launch_bounds__(256) void conv_rope_cache_kernel(
       a[i] = conv_at(col0 + 2 * pi);
       if (2 * pi + 1 < width) bb[i] = conv_at(col0 + 2 * pi + 1);
       if (!is_v && pi < pairs) {
-        const float ang = fpos * freq[pi];
-        const float cs = cosf(ang) * amp, sn = sinf(ang) * amp;
+        float cs, sn;
+        if (rot_table) {   // (the same two values, computed once per token by rotation_table_kernel)
+          cs = rot_table[t * rot_stride(pairs) + 2 * pi];
+          sn = rot_table[t * rot_stride(pairs) + 2 * pi + 1];
+        } else {
+          const float ang = fpos * freq[pi];
+          cs = cosf(ang) * amp;
+          sn = sinf(ang) * amp;
+        }
         const float x0 = a[i], x1 = bb[i];
         a[i] = x0 * cs - x1 * sn;
         bb[i] = x1 * cs + x0 * sn;
@@ -197,12 +210,12 @@ __device__ __forceinline__ float row16_sum(float v) {
 // its rows take in step: the tap weights and the bias of an item are fetched once for the sixteen tokens, and the rows a tap
 // reads are the neighbouring rows' own.  Lane r of a row owns the 16-byte pieces r, r + 16, .. of the head (up to four: widths
 // <= 512 sixteen-bit / 256 fp32 channels, multiples of 8 / 4; how many is a template constant, as are the taps (0 .. 4), so a
-// piece's tap weights sit in registers.  A token's cos / sin are computed once per workgroup, into LDS [16][2][pairs].  The same sums in
-// the same order as the plain form.
+// piece's tap weights sit in registers.  A token's cos / sin come from the step's rotation table.  The same sums in the
+// same order as the plain form.
 template <int DT, int TAPS, int NPC>   // NPC: 16-byte pieces per lane (1, 2 or 4)
 __global__ __launch_bounds__(256) void conv_rope_cache_vec_kernel(
     const void* __restrict__ qkv, int64_t ld, const void* __restrict__ bias, const void* __restrict__ conv_w,
-    void* __restrict__ conv_state, int64_t state_half, const float* __restrict__ freq, int pairs, float amp, int unit_norm,
+    void* __restrict__ conv_state, int64_t state_half, const float* __restrict__ rot_table, int pairs, int unit_norm,
     float eps, const void* __restrict__ v_src, int64_t v_src_stride, const void* __restrict__ v_lam,
     const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ select,
     const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_first_pos, const int32_t* __restrict__ seq_slot,
@@ -213,7 +226,6 @@ __global__ __launch_bounds__(256) void conv_rope_cache_vec_kernel(
   struct alignas(16) Piece { elem e[EPC]; };
   constexpr int BACK = TAPS > 1 ? TAPS - 1 : 0;
   constexpr int WN = TAPS > 0 ? TAPS : 1;
-  extern __shared__ float rot_cs[];   // [16 tokens][cos | sin][pairs], times amp
   const int items = heads + 2 * kv_heads;
   const int trow = threadIdx.x >> 4, r = threadIdx.x & 15;
   const int64_t t = (int64_t)blockIdx.x * 16 + trow;
@@ -224,14 +236,7 @@ __global__ __launch_bounds__(256) void conv_rope_cache_vec_kernel(
   const int in_run = pos - first;
   const int item_lo = blockIdx.y * items_per_wg;
   const int item_hi = item_lo + items_per_wg < items ? item_lo + items_per_wg : items;
-  float* my_cs = rot_cs + (int64_t)trow * 2 * pairs;
-  for (int i = r; i < pairs; i += 16) {
-    float sn, cs;
-    sincosf((float)pos * freq[i], &sn, &cs);
-    my_cs[i] = cs * amp;
-    my_cs[pairs + i] = sn * amp;
-  }
-  __builtin_amdgcn_wave_barrier();   // (written and read by the lanes of one row, which share a wave)
+  const float* my_cs = rot_table + t * rot_stride(pairs);   // (cos, sin) of the token's angles, times the amplitude
   const bool last_of_run = t == seq_start[b + 1] - 1;
   float lam = 0.f;
   if (v_src) lam = ldv<DT>(v_lam, 0);
@@ -277,17 +282,6 @@ __global__ __launch_bounds__(256) void conv_rope_cache_vec_kernel(
             else bv[e] = to_f32<DT>(braw.e[e]);
           }
         }
-        float w[WN][EPC];
-        if constexpr (TAPS > 0) {
-#pragma unroll
-          for (int k = 0; k < TAPS; ++k) {
-#pragma unroll
-            for (int e = 0; e < EPC; ++e) {
-              if constexpr (DT == LL_F32) w[k][e] = wraw[k].e[e];
-              else w[k][e] = to_f32<DT>(wraw[k].e[e]);
-            }
-          }
-        }
 #pragma unroll
         for (int jt = 0; jt < WN; ++jt) {
           const bool seen = WN - 1 - jt <= pos;
@@ -297,20 +291,29 @@ __global__ __launch_bounds__(256) void conv_rope_cache_vec_kernel(
             if constexpr (DT == LL_F32) u = raw[jt].e[e];
             else u = to_f32<DT>(raw[jt].e[e]);
             if (bias) u += bv[e];
-            if constexpr (TAPS > 0) {
+            if constexpr (TAPS > 0) {   // (weights widened where they are used: fewer live registers)
               const int flat = e * TAPS + jt;
-              acc[e] += w[flat / EPC][flat % EPC] * (seen ? u : 0.f);
+              float wt;
+              if constexpr (DT == LL_F32) wt = wraw[flat / EPC].e[flat % EPC];
+              else wt = to_f32<DT>(wraw[flat / EPC].e[flat % EPC]);
+              acc[e] += wt * (seen ? u : 0.f);
             } else {
               acc[e] = u;
             }
           }
         }
-        if (!is_v) {
+        if (!is_v && pc * (EPC / 2) < pairs) {
+          float rot[EPC];   // (cos, sin) of this piece's pairs: EPC floats at pc * EPC, inside the padded row
+#pragma unroll
+          for (int k = 0; k < EPC / 4; ++k) {
+            const f32x4 v4 = *reinterpret_cast<const f32x4*>(my_cs + pc * EPC + 4 * k);
+            rot[4 * k] = v4[0]; rot[4 * k + 1] = v4[1]; rot[4 * k + 2] = v4[2]; rot[4 * k + 3] = v4[3];
+          }
 #pragma unroll
           for (int m = 0; m < EPC / 2; ++m) {
             const int pi = pc * (EPC / 2) + m;
             if (pi < pairs) {
-              const float cs = my_cs[pi], sn = my_cs[pairs + pi];
+              const float cs = rot[2 * m], sn = rot[2 * m + 1];
               const float x0 = acc[2 * m], x1 = acc[2 * m + 1];
               acc[2 * m] = x0 * cs - x1 * sn;
               acc[2 * m + 1] = x1 * cs + x0 * sn;
@@ -583,8 +586,33 @@ extern "C" int ll_qk_norm_cache(const void* qkv, int64_t ld, const void* q_w, co
   return LL_LAUNCH_CHECK();
 }
 
+namespace {
+// one thread per (token, pair): out[t][i] = (cos(pos * f_i) * amp, sin(pos * f_i) * amp); rows of rot_stride(pairs) floats
+__global__ __launch_bounds__(256) void rotation_table_kernel(const int32_t* __restrict__ tok_pos, const float* __restrict__ freq,
+                                                             int pairs, float amp, float* __restrict__ out, int64_t n) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= n * pairs) return;
+  const int64_t t = idx / pairs;
+  const int i = (int)(idx - t * pairs);
+  float sn, cs;
+  sincosf((float)tok_pos[t] * freq[i], &sn, &cs);   // (one argument reduction for both)
+  out[t * rot_stride(pairs) + 2 * i] = cs * amp;
+  out[t * rot_stride(pairs) + 2 * i + 1] = sn * amp;
+}
+}  // namespace
+
+extern "C" int ll_rotation_table(const int32_t* tok_pos, const float* freq, int64_t pairs, float amp, float* out, int64_t n,
+                                 void* stream) {
+  if (n < 0 || pairs < 1 || pairs > 4096) return LL_ERR_SHAPE;
+  if (n == 0) return LL_OK;
+  if (!tok_pos || !freq || !out) return LL_ERR_ARG;
+  rotation_table_kernel<<<dim3((unsigned)((n * pairs + 255) / 256)), 256, 0, (hipStream_t)stream>>>(tok_pos, freq, (int)pairs, amp, out, n);
+  return LL_LAUNCH_CHECK();
+}
+
 extern "C" int ll_conv_rope_cache(const void* qkv, int64_t ld, const void* bias, const void* conv_w, int64_t taps, void* conv_state,
-                                  int64_t state_half, const float* freq, int64_t pairs, float amp, int unit_norm, float eps,
+                                  int64_t state_half, const float* freq, int64_t pairs, float amp, const float* rot_table,
+                                  int unit_norm, float eps,
                                   const void* v_src, int64_t v_src_stride, const void* v_lam, const int32_t* tok_seq,
                                   const int32_t* tok_pos, const int32_t* select, const int32_t* seq_start,
                                   const int32_t* seq_first_pos, const int32_t* seq_slot, const int32_t* seq_parity, void* q_out,
@@ -596,18 +624,18 @@ extern "C" int ll_conv_rope_cache(const void* qkv, int64_t ld, const void* bias,
     return LL_ERR_SHAPE;
   if (n == 0) return LL_OK;
   if (!qkv || !tok_seq || !tok_pos || !select || !seq_start || !seq_first_pos || !seq_slot || !seq_parity || !q_out || !k_cache ||
-      !v_cache || (taps > 0 && !conv_w) || (taps > 1 && !conv_state) || (pairs > 0 && !freq) || (v_src && !v_lam))
+      !v_cache || (taps > 0 && !conv_w) || (taps > 1 && !conv_state) || (pairs > 0 && !freq && !rot_table) || (v_src && !v_lam))
     return LL_ERR_ARG;
   const int64_t waves = n * (heads + 2 * kv_heads);
   const dim3 grid((unsigned)((waves + 3) / 4));
   const int64_t widest = dk > dv ? dk : dv;
   hipStream_t st = (hipStream_t)stream;
 #define LL_CR_ARGS                                                                                                              \
-  qkv, ld, bias, conv_w, (int)taps, conv_state, state_half, freq, (int)pairs, amp, unit_norm, eps, v_src, v_src_stride, v_lam, tok_seq, \
+  qkv, ld, bias, conv_w, (int)taps, conv_state, state_half, freq, (int)pairs, amp, rot_table, unit_norm, eps, v_src, v_src_stride, v_lam, tok_seq, \
       tok_pos, select, seq_start, seq_first_pos, seq_slot, seq_parity, q_out, k_cache, v_cache, n, (int)heads, (int)kv_heads, (int)dk, \
       (int)dv
   const int epc = dtype == LL_F32 ? 4 : 8;
-  const bool vec = taps <= 4 && dk % epc == 0 && dv % epc == 0 && ld % epc == 0 && widest <= 64 * epc && ll_aligned16(qkv) &&
+  const bool vec = (pairs == 0 || (rot_table && ll_aligned16(rot_table))) && taps <= 4 && dk % epc == 0 && dv % epc == 0 && ld % epc == 0 && widest <= 64 * epc && ll_aligned16(qkv) &&
                    ll_aligned16(q_out) && ll_aligned16(k_cache) && ll_aligned16(v_cache) && (!bias || ll_aligned16(bias)) &&
                    (!conv_w || ll_aligned16(conv_w)) && (taps <= 1 || ll_aligned16(conv_state)) &&
                    (!v_src || (ll_aligned16(v_src) && v_src_stride % epc == 0));
@@ -616,9 +644,9 @@ extern "C" int ll_conv_rope_cache(const void* qkv, int64_t ld, const void* bias,
     const int64_t tiles = (n + 15) / 16, items = heads + 2 * kv_heads;
     const int ipw = tiles * ((items + 3) / 4) >= 1024 ? 4 : 1;
     const dim3 grid_v((unsigned)tiles, (unsigned)((items + ipw - 1) / ipw));
-    const size_t lds_v = sizeof(float) * 16 * 2 * (size_t)(pairs > 0 ? pairs : 1);
+    const size_t lds_v = 0;
 #define LL_CRV_ARGS                                                                                                              \
-  qkv, ld, bias, conv_w, conv_state, state_half, freq, (int)pairs, amp, unit_norm, eps, v_src, v_src_stride, v_lam, tok_seq, tok_pos, \
+  qkv, ld, bias, conv_w, conv_state, state_half, rot_table, (int)pairs, unit_norm, eps, v_src, v_src_stride, v_lam, tok_seq, tok_pos, \
       select, seq_start, seq_first_pos, seq_slot, seq_parity, q_out, k_cache, v_cache, n, (int)heads, (int)kv_heads, (int)dk, (int)dv, ipw
     const int npc = widest <= 16 * epc ? 1 : widest <= 32 * epc ? 2 : 4;
 #define CALL_N(DT, T)                                                                                            \

@@ -11,7 +11,7 @@ this drives the layered models (model_layers.py): one flat token array, no paddi
 from __future__ import annotations
 
 from collections.abc import Sequence
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 
 import torch
 
@@ -37,6 +37,7 @@ class RaggedStep:
     longest_run: int = 0       # most tokens a sequence brings (host copy; 0: not known)
     longest_context: int = 0   # longest sequence after this step (host copy; 0: not known)
     all_start: bool = False    # every sequence of the step starts at position 0 (host copy; False: not known)
+    shared: dict = field(default_factory=dict, compare=False, repr=False)   # what layers of one forward pass compute once (rotation tables)
 
     @property
     def seq_req(self) -> torch.Tensor:

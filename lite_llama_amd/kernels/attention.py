@@ -310,9 +310,22 @@ def qk_norm_cache(qkv, heads: int, kv_heads: int, dk: int, dv: int, q_weight, k_
 
 
 @torch.no_grad()
+def rotation_table(step, freq, pairs: int, amp: float = 1.0):
+    """fp32 ``[n, 2 * pairs4]`` (``pairs4``: ``pairs`` rounded up to a multiple of 4, the padding zero): per token of the step and
+    entry pair ``(cos(position * freq[i]) * amp, sin(position * freq[i]) * amp)``."""
+    L.require_cuda(freq)
+    if freq.dtype != torch.float32 or freq.numel() < pairs or not freq.is_contiguous() or pairs < 1:
+        raise ValueError("rotation_table: fp32 frequencies, one per rotated pair")
+    out = torch.zeros(step.num_tokens, 2 * (-(-pairs // 4) * 4), dtype=torch.float32, device=freq.device)
+    L.check(L.lib().ll_rotation_table(step.tok_pos.data_ptr(), freq.data_ptr(), int(pairs), float(amp), out.data_ptr(), step.num_tokens,
+                                      L.stream_ptr()), "rotation_table")
+    return out
+
+
+@torch.no_grad()
 def conv_rope_cache(qkv, heads: int, kv_heads: int, dk: int, dv: int, step, k_cache, v_cache, *, bias=None, conv_weight=None,
                     conv_state=None, freq=None, pairs: int = 0, amp: float = 1.0, unit_norm: bool = False, eps: float = 0.0,
-                    v_source=None, v_blend=None):
+                    v_source=None, v_blend=None, rot_table=None):
     """Fused projection rows ``[q | k | v]`` -> queries ``[n, heads, dk]``; keys and values land in the cache rows
     ``step.select``.  Channel by channel, in fp32: ``+ bias``; a causal convolution over the sequence's positions with
     ``conv_weight [channels, taps]`` (``y_t = sum_j w[:, j] u_(t - taps + 1 + j)``, zeros in front of position 0), the raw rows of
@@ -320,7 +333,8 @@ def conv_rope_cache(qkv, heads: int, kv_heads: int, dk: int, dv: int, step, k_ca
     sequence's parity is read, the other written); entry pairs ``(2i, 2i + 1)``, ``i < pairs``, of every q / k head rotated by
     ``position * freq[i]`` with cos / sin times ``amp``; q / k heads divided by ``sqrt(mean + eps)`` when ``unit_norm``; values
     become ``(1 - b) v + b v_source[select]`` when ``v_source [rows, kv_heads, dv]`` (another layer's value cache) and the
-    one-element tensor ``v_blend`` are given."""
+    one-element tensor ``v_blend`` are given.  ``rot_table``: :func:`rotation_table` of this step for these frequencies (made
+    here when absent; layers that rotate alike share one)."""
     L.require_cuda(qkv, k_cache, v_cache, bias, conv_weight, conv_state, freq, v_source, v_blend)
     n, dt = qkv.shape[0], qkv.dtype
     channels = (heads + kv_heads) * dk + kv_heads * dv
@@ -345,11 +359,17 @@ def conv_rope_cache(qkv, heads: int, kv_heads: int, dk: int, dv: int, step, k_ca
                                  or tuple(v_source.shape[1:]) != (kv_heads, dv) or not v_source.is_contiguous()
                                  or v_source.shape[0] != v_cache.shape[0]):
         raise ValueError("conv_rope_cache: the blended values are another cache of this one's shape, with a one-element weight")
+    if pairs and rot_table is None:
+        rot_table = rotation_table(step, freq, pairs, amp)
+    if pairs and (rot_table.dtype != torch.float32 or tuple(rot_table.shape) != (n, 2 * (-(-pairs // 4) * 4))
+                  or not rot_table.is_contiguous()):
+        raise ValueError("conv_rope_cache: the rotation table is what rotation_table() returns for this step and these pairs")
     q = torch.empty(n, heads, dk, dtype=dt, device=qkv.device)
     half = conv_state[0].numel() if (conv_state is not None and taps > 1) else 0
     L.check(L.lib().ll_conv_rope_cache(
         qkv.data_ptr(), qkv.stride(0), L.ptr(bias), L.ptr(conv_weight), taps, L.ptr(conv_state) if taps > 1 else 0, half,
-        L.ptr(freq) if pairs else 0, int(pairs), float(amp), 1 if unit_norm else 0, float(eps), L.ptr(v_source),
+        L.ptr(freq) if pairs else 0, int(pairs), float(amp), L.ptr(rot_table) if pairs else 0, 1 if unit_norm else 0, float(eps),
+        L.ptr(v_source),
         v_source.stride(0) if v_source is not None else 0, L.ptr(v_blend) if v_source is not None else 0, step.tok_seq.data_ptr(),
         step.tok_pos.data_ptr(), step.select.data_ptr(), step.seq_start.data_ptr(), step.seq_first_pos.data_ptr(),
         step.seq_slot.data_ptr(), step.seq_parity.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), n, heads,

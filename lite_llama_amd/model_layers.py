@@ -44,7 +44,7 @@ import torch.nn.functional as F
 
 from .distributed.parallel_state import get_tp_world_size
 from .kernels.activations import xielu
-from .kernels.attention import conv_rope_cache, latent_kv_prep, qk_norm_cache, ragged_attention, rotate_pairs
+from .kernels.attention import conv_rope_cache, latent_kv_prep, qk_norm_cache, ragged_attention, rotate_pairs, rotation_table
 from .kernels.fused_moe import group_router, sparse_glu_experts
 from .kernels.norm_act import (GatedUpdate, SummedUpdate, add_rmsnorm_shift, cast_pair, embed_pair, gated_group_norm, glu_act,
                                residual_set, softcap_)
@@ -567,11 +567,20 @@ class ConvRotaryAttention(nn.Module):
         if s.unit_sink and (self._sink is None or self._sink.device != h.device or self._sink.dtype != h.dtype):
             self._sink = torch.zeros(s.heads, dtype=h.dtype, device=h.device)
         source = cache.value_source[run]
+        table = None
+        if self.pairs:   # cos / sin per token: once per step for all layers that rotate alike
+            key = ("rotation", self.pairs, self.amp, tuple(self._freq_values))
+            shared = getattr(step, "shared", None)
+            table = shared.get(key) if shared is not None else None
+            if table is None:
+                table = rotation_table(step, self._freq, self.pairs, self.amp)
+                if shared is not None:
+                    shared[key] = table
         q = conv_rope_cache(rows, s.heads, s.kv_heads, s.dim, s.vdim, step, k_cache, v_cache, bias=self.qkv_bias,
                             conv_weight=self.conv_weight, conv_state=cache.conv[run], freq=self._freq, pairs=self.pairs,
                             amp=self.amp, unit_norm=s.unit_norm, eps=self.eps,
                             v_source=cache.kv_buffer[source][1] if source is not None else None,
-                            v_blend=self.value_blend if source is not None else None)
+                            v_blend=self.value_blend if source is not None else None, rot_table=table)
         o = ragged_attention(q, k_cache, v_cache, s.scale, step, token_table, sink=self._sink if s.unit_sink else None,
                              window=s.window, keep_first=s.keep_first, out=out)
         return o, (rows[:, self.channels:] if self.extra else None)
