@@ -22,7 +22,7 @@ from .rukedra_bench import _step_of
 def kernel_table(dev, dtype, width, heads, kv_heads, dim, vdim, taps, rot, window, keep, ff, experts, top, eff, buckets,
                  prefill=(8, 512), decode=(32, 1024)):
     from lite_llama_amd.kernels import flash_attention2_no_pad, flash_decoding, skip_rmsnorm, swiglu_forward
-    from lite_llama_amd.kernels.attention import conv_rope_cache, ragged_attention
+    from lite_llama_amd.kernels.attention import conv_rope_cache, ragged_attention, rotation_table
     from lite_llama_amd.kernels.fused_moe import fused_moe, group_router, moe_route_topk, sparse_glu_experts
     from lite_llama_amd.kernels.norm_act import SummedUpdate, add_rmsnorm_shift, embed_pair, glu_act, rope_and_cache
 
@@ -74,8 +74,13 @@ def kernel_table(dev, dtype, width, heads, kv_heads, dim, vdim, taps, rot, windo
         state = torch.zeros(2, batch, taps - 1, channels, device=dev, dtype=dtype)
         freq = torch.rand(rot // 2, device=dev)
         lam = torch.tensor([0.4], device=dev).to(dtype)
+        t_tab = _time(lambda: rotation_table(step, freq, rot // 2, 1.1))
+        out.append(dict(_entry("rotation_table (cos / sin per token and pair: once per step for all layers)", t_tab,
+                               n * rot * 4, 0), phase=phase))
+        tab = rotation_table(step, freq, rot // 2, 1.1)
         t_new = _time(lambda: conv_rope_cache(gu, heads, kv_heads, dim, vdim, step, kc, vc, bias=bias, conv_weight=cw, conv_state=state,
-                                              freq=freq, pairs=rot // 2, amp=1.1, unit_norm=True, eps=1e-6, v_source=src, v_blend=lam))
+                                              freq=freq, pairs=rot // 2, amp=1.1, unit_norm=True, eps=1e-6, v_source=src, v_blend=lam,
+                                              rot_table=tab))
         hd = 128
         qh = torch.randn(n, heads, hd, device=dev).to(h16)
         kvh = torch.randn(n, 2 * kv_heads, hd, device=dev).to(h16)

@@ -622,7 +622,7 @@ int ll_ragged_attention(const void* q, const void* k_cache, const void* v_cache,
  * lam v_src[select[t]] when v_src (rows of stride v_src_stride; lam = *v_lam) is given.  q -> q_out [n, heads, dk]; k, v ->
  * cache rows select[t]. */
 /* out [n][2 * pairs4] (fp32), pairs4 = pairs rounded up to a multiple of 4: entry pair i of token t at [t][2 i] =
- * (cos(tok_pos[t] * freq[i]) * amp, sin(tok_pos[t] * freq[i]) * amp); the padding is not written. */
+ * (cos(tok_pos[t] * freq[i]) * amp, sin(tok_pos[t] * freq[i]) * amp); the padding is zero. */
 int ll_rotation_table(const int32_t* tok_pos, const float* freq, int64_t pairs, float amp, float* out, int64_t n, void* stream);
 int ll_conv_rope_cache(const void* qkv, int64_t ld, const void* bias, const void* conv_w, int64_t taps, void* conv_state,
                        int64_t state_half, const float* freq, int64_t pairs, float amp, const float* rot_table,

@@ -591,9 +591,15 @@ namespace {
 __global__ __launch_bounds__(256) void rotation_table_kernel(const int32_t* __restrict__ tok_pos, const float* __restrict__ freq,
                                                              int pairs, float amp, float* __restrict__ out, int64_t n) {
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= n * pairs) return;
-  const int64_t t = idx / pairs;
-  const int i = (int)(idx - t * pairs);
+  const int padded = (int)(rot_stride(pairs) / 2);
+  if (idx >= n * padded) return;
+  const int64_t t = idx / padded;
+  const int i = (int)(idx - t * padded);
+  if (i >= pairs) {   // the padding reads as zeros
+    out[t * rot_stride(pairs) + 2 * i] = 0.f;
+    out[t * rot_stride(pairs) + 2 * i + 1] = 0.f;
+    return;
+  }
   float sn, cs;
   sincosf((float)tok_pos[t] * freq[i], &sn, &cs);   // (one argument reduction for both)
   out[t * rot_stride(pairs) + 2 * i] = cs * amp;
@@ -606,7 +612,8 @@ extern "C" int ll_rotation_table(const int32_t* tok_pos, const float* freq, int6
   if (n < 0 || pairs < 1 || pairs > 4096) return LL_ERR_SHAPE;
   if (n == 0) return LL_OK;
   if (!tok_pos || !freq || !out) return LL_ERR_ARG;
-  rotation_table_kernel<<<dim3((unsigned)((n * pairs + 255) / 256)), 256, 0, (hipStream_t)stream>>>(tok_pos, freq, (int)pairs, amp, out, n);
+  rotation_table_kernel<<<dim3((unsigned)((n * (rot_stride(pairs) / 2) + 255) / 256)), 256, 0, (hipStream_t)stream>>>(tok_pos, freq, (int)pairs,
+                                                                                                                 amp, out, n);
   return LL_LAUNCH_CHECK();
 }
 

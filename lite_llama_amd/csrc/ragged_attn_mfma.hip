@@ -354,18 +354,28 @@ __global__ __launch_bounds__(256) void ragged_attention_mfma_prefill4_kernel(
   for (int i = 0; i < NTM; ++i) ot[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   Q4 kr[KPASS], vr[VPASS];
+  int rk[KPASS], rv[VPASS];   // cache rows of the pieces this thread fetches next: read one tile ahead of the pieces themselves
   // piece i of a tile: key i / pieces-per-row, channels 8 (i % pieces-per-row); keys past the range load zeros
+#define LL_ROWS(P)                                                                                                 \
+  _Pragma("unroll") for (int u = 0; u < KPASS; ++u) {                                                              \
+    const int key = (tid + 256 * u) / kcpr;                                                                        \
+    rk[u] = (key < 32 && (P) + key < k_hi) ? table[(P) + key] : 0;                                                 \
+  }                                                                                                                \
+  if (!shared_kv) _Pragma("unroll") for (int u = 0; u < VPASS; ++u) {                                              \
+    const int key = (tid + 256 * u) / vcpr;                                                                        \
+    rv[u] = (key < 32 && (P) + key < k_hi) ? table[(P) + key] : 0;                                                 \
+  }
 #define LL_FETCH(P)                                                                                                \
   _Pragma("unroll") for (int u = 0; u < KPASS; ++u) {                                                              \
     const int i = tid + 256 * u, key = i / kcpr, piece = i - key * kcpr;                                           \
     kr[u] = (key < 32 && (P) + key < k_hi)                                                                         \
-                ? *reinterpret_cast<const Q4*>(k_cache + (int64_t)table[(P) + key] * k_stride + (int64_t)g * dk + 8 * piece) \
+                ? *reinterpret_cast<const Q4*>(k_cache + (int64_t)rk[u] * k_stride + (int64_t)g * dk + 8 * piece)  \
                 : Q4{0, 0, 0, 0};                                                                                  \
   }                                                                                                                \
   if (!shared_kv) _Pragma("unroll") for (int u = 0; u < VPASS; ++u) {                                              \
     const int i = tid + 256 * u, key = i / vcpr, piece = i - key * vcpr;                                           \
     vr[u] = (key < 32 && (P) + key < k_hi)                                                                         \
-                ? *reinterpret_cast<const Q4*>(v_cache + (int64_t)table[(P) + key] * v_stride + (int64_t)g * dv + 8 * piece) \
+                ? *reinterpret_cast<const Q4*>(v_cache + (int64_t)rv[u] * v_stride + (int64_t)g * dv + 8 * piece)  \
                 : Q4{0, 0, 0, 0};                                                                                  \
   }
 #define LL_STAGE()                                                                           \
@@ -377,13 +387,18 @@ __global__ __launch_bounds__(256) void ragged_attention_mfma_prefill4_kernel(
     const int i = tid + 256 * u, key = i / vcpr, piece = i - key * vcpr;                     \
     if (key < 32) *reinterpret_cast<Q4*>(&lds_v[key * VSTR + 8 * piece]) = vr[u];            \
   }
+  LL_ROWS(k_first_wg)
   LL_FETCH(k_first_wg)
+  LL_ROWS(next_tile(k_first_wg))   // (past the range: nothing is read)
   __syncthreads();   // the zero fill is complete
   LL_STAGE()
   __syncthreads();
   for (int p0 = k_first_wg, p1; p0 < k_hi; p0 = p1) {
     p1 = next_tile(p0);
-    if (p1 < k_hi) { LL_FETCH(p1) }
+    if (p1 < k_hi) {
+      LL_FETCH(p1)
+      LL_ROWS(next_tile(p1))
+    }
     if (wave_on && p0 < k_hi_w && (p0 + 32 > k_lo_w || p0 < keep_first)) {
       f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -448,6 +463,7 @@ __global__ __launch_bounds__(256) void ragged_attention_mfma_prefill4_kernel(
     if (p1 < k_hi) { LL_STAGE() }
     __syncthreads();
   }
+#undef LL_ROWS
 #undef LL_FETCH
 #undef LL_STAGE
   if (!valid) return;

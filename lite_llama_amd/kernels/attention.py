@@ -316,7 +316,7 @@ def rotation_table(step, freq, pairs: int, amp: float = 1.0):
     L.require_cuda(freq)
     if freq.dtype != torch.float32 or freq.numel() < pairs or not freq.is_contiguous() or pairs < 1:
         raise ValueError("rotation_table: fp32 frequencies, one per rotated pair")
-    out = torch.zeros(step.num_tokens, 2 * (-(-pairs // 4) * 4), dtype=torch.float32, device=freq.device)
+    out = torch.empty(step.num_tokens, 2 * (-(-pairs // 4) * 4), dtype=torch.float32, device=freq.device)
     L.check(L.lib().ll_rotation_table(step.tok_pos.data_ptr(), freq.data_ptr(), int(pairs), float(amp), out.data_ptr(), step.num_tokens,
                                       L.stream_ptr()), "rotation_table")
     return out

@@ -56,8 +56,8 @@ CONFIGS = {
                     attention(2, 2, 32, 24, 2, 6, 11, 16, v_mix=False, mlp=moe(8, 3, 8), original=512),
                     attention(20, 1, 8, 8, 6, 30, 2, 4, mlp=moe(2, 1, 16))], width=64, vocab=71, buckets=5, mul_prev=1, mul_cur=1),
     # everything that can be 1: one head of one pair, one tap, a window of one key plus one kept key, one expert of one, one
-    # bucket, one layer
-    "one": config([attention(1, 1, 2, 1, 1, 1, 1, 2, mlp=moe(1, 1, 8), scale=1.0)], width=16, vocab=11, buckets=1, mul_prev=3,
+    # bucket, one layer; a width that is no multiple of 4 (rows off every 8- and 16-byte border)
+    "one": config([attention(1, 1, 2, 1, 1, 1, 1, 2, mlp=moe(1, 1, 8), scale=1.0)], width=18, vocab=11, buckets=1, mul_prev=3,
                   mul_cur=5, scale=2.0, logit_scale=1.5),
 }
 
