@@ -565,3 +565,62 @@ def test_command_line_generate_and_trace_replay(tmp_path_factory, tmp_path):
     _close(read(1), lb[[5]], 2e-5)
     assert not (out / "2.f32").exists()
     _close(read(3), torch.stack([la[30], lb[5]]), 2e-5)
+
+
+def _random_config(seed):
+    """A configuration drawn from the whole range the reader takes: head counts and widths with and without the matrix-core
+    forms' multiples, 1 - 6 taps or none, windows from 1 key to longer than the prompt, kept keys from none to more than the
+    window, rotations of a part or all of a head with and without scaling, every feed-forward kind in any order, blending
+    layers anywhere."""
+    import random
+
+    r = random.Random(seed)
+    kv = r.choice([1, 2, 3])
+    dv = r.choice([8, 16, 24, 10, 48])
+    layers = []
+    for _ in range(r.randint(1, 4)):
+        mixes = r.random() < 0.7
+        g = kv if mixes else r.choice([1, 2])
+        heads = g * r.choice([1, 2, 4, 5])
+        dim = r.choice([8, 16, 32, 64, 12, 20, 128])
+        vdim = dv if mixes else r.choice([8, 12, 32])
+        dims = r.choice([dim, dim // 2, 2, max(2, (dim // 4) * 2)])
+        kind = r.choice(["dense", "moe", None])
+        experts = r.randint(1, 9)
+        mlp = T.dense(r.choice([16, 40, 44]), limit=r.choice([0.5, 2.0, 30.0])) if kind == "dense" else \
+            T.moe(experts, r.randint(1, experts), r.choice([8, 12, 24])) if kind == "moe" else None
+        layers.append(T.attention(heads, g, dim, vdim, r.choice([None, 1, 2, 3, 4, 6]), r.choice([1, 3, 8, 17, 40, 64, 200]),
+                                  r.choice([0, 0, 1, 2, 5, 33, 70]), dims, v_mix=mixes, mlp=mlp, scaled=r.random() < 0.7,
+                                  base=r.choice([100.0, 10000.0]), factor=r.choice([2.0, 4.0, 16.0]), original=r.choice([16, 64, 1024]),
+                                  scale=r.choice([0.5, 1.0, 2.0]) * dim ** -0.5 * 4))
+    return T.config(layers, width=r.choice([32, 48, 60, 88]), vocab=r.randint(20, 300), buckets=r.randint(1, 500),
+                    mul_prev=r.randint(0, 1000), mul_cur=r.randint(1, 1000), scale=r.choice([1.0, 0.25, 3.0]),
+                    logit_scale=r.choice([1.0, 0.125, 5.0]), eps=r.choice([1e-5, 1e-6, 1e-3]))
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_configurations_whole_in_portions_decoded_and_side_by_side(tmp_path, seed):
+    from lite_llama_amd.executor.ragged import RaggedRunner
+    from lite_llama_amd.weights import load_pretrained
+    from oracle import fekanex as O
+
+    cfg = _random_config(seed)
+    tens = T.tensors(cfg, seed=seed)
+    model = load_pretrained(L.write(tmp_path / "m", cfg, tens), device=DEV, dtype=torch.float32)
+    a, b = L.prompt(cfg, 90, seed=seed), L.prompt(cfg, 37, seed=seed + 50)
+    wa, wb = O.forward(a, tens, cfg), O.forward(b, tens, cfg)
+    runner = RaggedRunner(model, 256, 3, block_size=16, device=DEV)
+    _close(_feed(runner, runner.admit(), a, [90]), wa, 3e-5)
+    _close(_feed(runner, runner.admit(), a, [2, 1, 7, 3, 1, 30, 1]), wa, 3e-5)
+    runner.release([0, 1])
+    sa, sb = runner.admit(), runner.admit()            # used slots and pages again, two requests side by side
+    got_a, got_b, ia, ib = [], [], 0, 0
+    for ca, cb in [(11, 1), (1, 2), (40, 1), (1, 20), (5, 1), (32, 12)]:
+        out = runner.step([(sa, a[ia:ia + ca]), (sb, b[ib:ib + cb])], list(range(ca + cb)))
+        got_a.append(out[:ca])
+        got_b.append(out[ca:])
+        ia, ib = ia + ca, ib + cb
+    assert ia == 90 and ib == 37
+    runner.check_errors()
+    _close(torch.cat(got_a), wa, 3e-5)
+    _close(torch.cat(got_b), wb, 3e-5)
