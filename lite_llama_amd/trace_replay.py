@@ -68,6 +68,8 @@ def main(argv=None) -> int:
         for e in msg["entries"]:
             if e["id"] not in slots:
                 slots[e["id"]] = runner.admit()
+            if not e["tokens"]:
+                continue  # (admitted, brings nothing in this step)
             entries.append((slots[e["id"]], e["tokens"]))
             rows += [base + int(w) for w in e.get("want", [])]
             base += len(e["tokens"])
