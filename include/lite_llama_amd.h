@@ -649,11 +649,13 @@ int ll_ragged_attention_mfma(const void* q, const void* k_cache, const void* v_c
  * ll_gated_group_norm: with y: s = (sum of `parts` rows y[t][p][:] + shared_scale[t] * shared[t][:]) * sigmoid(gate[t][:] +
  * gate_bias) (shared, gate, gate_bias may be NULL; gate rows have stride gate_ld), x_out = x_in + groupnorm(s) * post_w, and,
  * when h_out is given, h_out = groupnorm(x_out) * next_w.  Without y: h_out = groupnorm(x_in) * next_w.  groupnorm: the row in
- * `groups` equal consecutive parts, each divided by sqrt(mean(part^2) + eps).  x_out may be x_in. */
+ * `groups` equal consecutive parts, each divided by sqrt(mean(part^2) + eps).  x_out may be x_in.  y_bias [width] (or NULL) is
+ * added to the summed rows (the bias of the projection that produced them).  h_out without next_w: the new residual itself in
+ * the storage dtype (a sublayer that reads the residual stream without a norm in front). */
 int ll_gated_group_norm(const float* x_in, float* x_out, void* h_out, const void* y, int64_t parts, const void* shared,
                         const float* shared_scale, const void* gate, int64_t gate_ld, const void* gate_bias,
                         const void* post_w, const void* next_w, int64_t n, int64_t width, int64_t groups, float eps,
-                        int dtype, void* stream);
+                        const void* y_bias, int dtype, void* stream);
 /* out [n, ff] (rows of stride out_ld) = act(gate[t][j]) * up[t][j], gate / up rows of stride gate_ld / up_ld; kind 0: silu,
  * 1: gelu (tanh form), 2: sigmoid, 3: clamped -- g = min(gate, p0), u = clamp(up, -p0, p0), g sigmoid(p1 g) (u + 1). */
 int ll_glu_act(void* out, int64_t out_ld, const void* gate, int64_t gate_ld, const void* up, int64_t up_ld, int64_t n,
@@ -690,21 +692,61 @@ int ll_rotate_pairs(const void* q, int64_t q_tok_stride, int64_t q_head_stride, 
  * of its two best, the best group_keep groups stay eligible; ids [n, top] / weights [n, top] (fp32) = the top eligible experts
  * by score and score / (sum + 1e-20) * route_scale.  w_extra [width] (or NULL): extra_scale[t] = sigmoid(w_extra . h).
  * logits: fp32 scratch [n][experts + (w_extra ? 1 : 0)].  scoring 1: no sigmoid and no groups -- the `top` largest logits
- * are chosen and their weights are the softmax over the chosen logits alone (times route_scale).
+ * are chosen and their weights are the softmax over the chosen logits alone (times route_scale).  scoring 2: scores =
+ * softmax over all logits; ranked by score + correction[e] (storage dtype, or NULL); weights = the chosen scores themselves;
+ * the last `identity` experts return the token's own row: their slots keep ids >= experts - identity (never placed by
+ * ll_moe_sort over the experts that have weights) and extra_scale[t] receives the sum of their scores.
  * ll_moe_sort: slots sorted by expert in blocks of `block` = ll_moe_rows_block(...) rows, 32 or 128 (counts: int32 scratch
  * [experts]; sorted [num_slots + experts (block - 1)], block_expert [ceil(that / block)], num_post [1]).
  * ll_moe_rows_gemm: glu != 0: w [experts][2 N][K] (gate rows, then up rows), out[slot] = silu(a Wg^T) * (a Wu^T) with
- * a = row slot / a_div; glu == 0: w [experts][N][K], out[slot] = (a W^T) * slot_weight[slot]. */
+ * a = row slot / a_div (glu == 2: g' sigmoid(1.702 g') (u' + 1) with g' = min(g, limit), u' = clamp(u, -limit, limit));
+ * glu == 0: w [experts][N][K], out[slot] = (a W^T) * slot_weight[slot]. */
 int ll_group_router(const void* h, int64_t h_ld, const void* w_router, const void* w_extra, int64_t n, int64_t width,
                     int64_t experts, int64_t top, int64_t group_count, int64_t group_keep, float route_scale, int scoring,
-                    int32_t* ids, float* weights, float* extra_scale, float* logits, int dtype, void* stream);
+                    int32_t* ids, float* weights, float* extra_scale, float* logits, const void* correction, int64_t identity,
+                    int dtype, void* stream);
 int64_t ll_moe_rows_block(int64_t num_slots, int64_t experts, int64_t width, int64_t ff, int dtype);
 int ll_moe_sort(const int32_t* ids, int64_t num_slots, int64_t experts, int64_t block, int32_t* counts, int32_t* sorted,
                 int32_t* block_expert, int32_t* num_post, void* stream);
 int ll_moe_rows_gemm(const void* a, int64_t a_ld, int64_t a_div, const void* w, int64_t w_stride_e, int64_t K, int64_t N,
                      int glu, const float* slot_weight, void* out, int64_t out_ld, const int32_t* sorted,
                      const int32_t* block_expert, const int32_t* num_post, int64_t num_slots, int64_t experts, int64_t block,
-                     int dtype, void* stream);
+                     float limit, int dtype, void* stream);
+
+/* ---- linear attention with a decay, and what stands around it (csrc/linear_mix.hip) -----------------------------------------
+ * ll_linear_scan: per head S_t = diag(a_t) S_(t-1) + k_t (b_t v_t)^T, o_t = S_t^T q_t (+ skip_h v_t), fp32 state
+ * [slots, heads, dk, dv]; value head h reads query / key head h / qk_rep of rows q / k (strides q_ld / k_ld), its values at
+ * columns h dv of rows v.  act != 0: q, k, v through silu first.  q times q_scale.  kind 0: a = head_decay[h] (fp32); kind 1:
+ * a = sigmoid(gate[t][h dk + i] + gate_bias[h dk + i])^inv_tau per key entry; kind 2: dt = softplus(dt[t][h] + dt_bias[h]),
+ * a = exp(-exp(a_log[h]) dt), b = dt, skip [heads] or NULL.  o: fp32 [n, heads dv].  A run that starts at position 0 starts
+ * from zeros.
+ * ll_gated_out_norm: o fp32 [n, width] -> RMS norm over `parts` equal consecutive parts, times w[(channel) mod w_len] (NULL:
+ * none), times act(gate) (gate_kind 0 none, 1 silu, 2 sigmoid; gate_first: before the norm), times out_scale -> out rows of
+ * stride out_ld.
+ * ll_conv_act: out = silu(bias + causal convolution over a sequence's positions of rows [n, >= channels] with w
+ * [channels, taps]); state [2][slots][taps - 1][channels] (storage dtype; halves of state_half elements) carries the raw rows of
+ * a sequence's last positions, double-buffered by seq_parity.
+ * ll_rownorm_rope_cache: rows [q | k | v]; q and k RMS-normed over their whole row times q_w / k_w (NULL: no norm), entry i <
+ * pairs of every head rotated with entry i + pairs by tok_pos * freq[i]; q -> q_out [n, heads, dk], k and value_scale * v ->
+ * cache rows select[t]. */
+int ll_linear_scan_supported(int64_t dk, int64_t dv);
+int ll_linear_scan(const void* q, int64_t q_ld, const void* k, int64_t k_ld, const void* v, int64_t v_ld, int64_t heads,
+                   int64_t dk, int64_t dv, int64_t qk_rep, int kind, int act, float q_scale, const float* head_decay,
+                   const void* gate, int64_t gate_ld, const void* gate_bias, float inv_tau, const void* dt, int64_t dt_ld,
+                   const void* dt_bias, const void* a_log, const void* skip, float* o, int64_t batch,
+                   const int32_t* seq_start, const int32_t* seq_first_pos, const int32_t* seq_slot, float* state,
+                   int dtype, void* stream);
+int ll_gated_out_norm(void* out, int64_t out_ld, const float* o, const void* gate, int64_t gate_ld, int gate_kind,
+                      int gate_first, const void* w, int64_t w_len, float eps, float out_scale, int64_t n, int64_t width,
+                      int64_t parts, int dtype, void* stream);
+int ll_conv_act(void* out, int64_t out_ld, const void* rows, int64_t ld, const void* w, const void* bias, int64_t channels,
+                int64_t taps, void* state, int64_t state_half, const int32_t* tok_seq, const int32_t* tok_pos,
+                const int32_t* seq_start, const int32_t* seq_first_pos, const int32_t* seq_slot, const int32_t* seq_parity,
+                int64_t n, int dtype, void* stream);
+int ll_rownorm_rope_cache(const void* rows, int64_t ld, const void* q_w, const void* k_w, float eps, const float* freq,
+                          int64_t pairs, float value_scale, const int32_t* tok_pos, const int32_t* select, void* q_out,
+                          void* k_cache, void* v_cache, int64_t n, int64_t heads, int64_t kv_heads, int64_t dk, int64_t dv,
+                          int dtype, void* stream);
 
 #ifdef __cplusplus
 }

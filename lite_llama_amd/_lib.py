@@ -124,17 +124,22 @@ SIGNATURES = {
     "ll_ragged_attention_mfma_supported": [L, L, I],
     "ll_ragged_attention_partition": [],
     "ll_ragged_attention_mfma": [P, P, P, P, L, P, P, P, P, F, P, L, L, L, L, I, P, L, L, L, L, L, L, L, L, L, I, P],
-    "ll_gated_group_norm": [P, P, P, P, L, P, P, P, L, P, P, P, L, L, L, F, I, P],
+    "ll_gated_group_norm": [P, P, P, P, L, P, P, P, L, P, P, P, L, L, L, F, P, I, P],
     "ll_glu_act": [P, L, P, L, P, L, L, L, I, F, F, I, P],
     "ll_softcap": [P, L, F, I, P],
     "ll_mingru_scan_scratch_floats": [L, L, L],
     "ll_mingru_scan": [P, P, P, L, P, P, P, L, L, P, P, P, P, L, P, I, P],
     "ll_latent_kv_prep": [P, L, L, L, L, P, F, P, L, F, P, P, P, L, L, L, P, P, L, I, P],
     "ll_rotate_pairs": [P, L, L, L, L, P, L, F, P, P, L, L, L, L, I, P],
-    "ll_group_router": [P, L, P, P, L, L, L, L, L, L, F, I, P, P, P, P, I, P],
+    "ll_group_router": [P, L, P, P, L, L, L, L, L, L, F, I, P, P, P, P, P, L, I, P],
     "ll_moe_rows_block": [L, L, L, L, I],
     "ll_moe_sort": [P, L, L, L, P, P, P, P, P],
-    "ll_moe_rows_gemm": [P, L, L, P, L, L, L, I, P, P, L, P, P, P, L, L, L, I, P],
+    "ll_moe_rows_gemm": [P, L, L, P, L, L, L, I, P, P, L, P, P, P, L, L, L, F, I, P],
+    "ll_linear_scan_supported": [L, L],
+    "ll_linear_scan": [P, L, P, L, P, L, L, L, L, L, I, I, F, P, P, L, P, F, P, L, P, P, P, P, L, P, P, P, P, I, P],
+    "ll_gated_out_norm": [P, L, P, P, L, I, I, P, L, F, F, L, L, L, I, P],
+    "ll_conv_act": [P, L, P, L, P, P, L, L, P, L, P, P, P, P, P, P, L, I, P],
+    "ll_rownorm_rope_cache": [P, L, P, P, F, P, L, F, P, P, P, P, P, L, L, L, L, L, I, P],
 }
 
 _RETURNS_I64 = {"ll_ragged_attention_partition", "ll_mingru_scan_scratch_floats", "ll_moe_rows_block", "ll_kv_alloc_scratch_bytes", "ll_tp_oneshot_flag_words", "ll_moe_router_workspace_floats", "ll_moe_align_workspace_ints"}

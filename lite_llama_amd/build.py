@@ -30,12 +30,13 @@ FLAGS += os.environ.get("LL_EXTRA_HIPCC_FLAGS", "").split()  # debug builds (e.g
 _NO_PACKED_FP32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 FILE_FLAGS = {"gemm_short.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"],
               "seq_mix.hip": _NO_PACKED_FP32, "ragged_attn.hip": _NO_PACKED_FP32, "ragged_attn_mfma.hip": _NO_PACKED_FP32,
-              "group_norm.hip": _NO_PACKED_FP32, "latent_attn.hip": _NO_PACKED_FP32, "moe_sparse.hip": _NO_PACKED_FP32}
+              "group_norm.hip": _NO_PACKED_FP32, "latent_attn.hip": _NO_PACKED_FP32, "moe_sparse.hip": _NO_PACKED_FP32,
+              "linear_mix.hip": _NO_PACKED_FP32}
 
 
 # part libraries: the sources ONE model family needs (a fresh checkout serving only that family builds nothing else)
 PARTS = {"ragged": ["seq_mix.hip", "ragged_attn.hip", "ragged_attn_mfma.hip", "group_norm.hip", "latent_attn.hip", "moe_sparse.hip",
-                    "kv_paged.hip", "kv_ops.hip", "sampler.hip"]}
+                    "linear_mix.hip", "kv_paged.hip", "kv_ops.hip", "sampler.hip"]}
 
 
 def flags_for(src: str) -> list[str]:

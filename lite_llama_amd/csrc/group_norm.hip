@@ -53,7 +53,7 @@ __global__ __launch_bounds__(256) void gated_group_norm_kernel(
     const float* x_in, float* x_out, void* __restrict__ h_out, const void* __restrict__ y, int parts,
     const void* __restrict__ shared, const float* __restrict__ shared_scale, const void* __restrict__ gate, int64_t gate_ld,
     const void* __restrict__ gate_bias, const void* __restrict__ post_w, const void* __restrict__ next_w, int width, int groups,
-    float eps) {
+    float eps, const void* __restrict__ y_bias) {
   constexpr bool EXACT = DT == LL_F32;
   __shared__ float red[4];
   const int64_t t = blockIdx.x;
@@ -66,6 +66,7 @@ __global__ __launch_bounds__(256) void gated_group_norm_kernel(
   auto branch = [&](int i) -> float {   // the sublayer's gated result at element i
     float s = 0.f;
     for (int p = 0; p < parts; ++p) s += ldv<DT>(y, (t * parts + p) * (int64_t)width + i);
+    if (y_bias) s += ldv<DT>(y_bias, i);
     if (shared) s += sscale * ldv<DT>(shared, t * (int64_t)width + i);
     if (gate) {
       float r = ldv<DT>(gate, t * gate_ld + i);
@@ -94,7 +95,8 @@ __global__ __launch_bounds__(256) void gated_group_norm_kernel(
       s2 = block_sum256(s2, red);
       if (h_out) {
         const float inv2 = 1.0f / sqrtf(s2 / (float)gs + eps);
-        for (int i = lo + tid; i < hi; i += 256) stv<DT>(h_out, t * (int64_t)width + i, xo[i] * inv2 * ldv<DT>(next_w, i));
+        for (int i = lo + tid; i < hi; i += 256)
+          stv<DT>(h_out, t * (int64_t)width + i, next_w ? xo[i] * inv2 * ldv<DT>(next_w, i) : xo[i]);
       }
     } else {
       float s2 = 0.f;
@@ -104,7 +106,8 @@ __global__ __launch_bounds__(256) void gated_group_norm_kernel(
       }
       s2 = block_sum256(s2, red);
       const float inv2 = 1.0f / sqrtf(s2 / (float)gs + eps);
-      for (int i = lo + tid; i < hi; i += 256) stv<DT>(h_out, t * (int64_t)width + i, xr[i] * inv2 * ldv<DT>(next_w, i));
+      for (int i = lo + tid; i < hi; i += 256)
+        stv<DT>(h_out, t * (int64_t)width + i, next_w ? xr[i] * inv2 * ldv<DT>(next_w, i) : xr[i]);
     }
   }
 }
@@ -116,7 +119,7 @@ __global__ __launch_bounds__(256) void gated_group_norm_cached_kernel(
     const float* x_in, float* x_out, void* __restrict__ h_out, const void* __restrict__ y, int parts,
     const void* __restrict__ shared, const float* __restrict__ shared_scale, const void* __restrict__ gate, int64_t gate_ld,
     const void* __restrict__ gate_bias, const void* __restrict__ post_w, const void* __restrict__ next_w, int width, int groups,
-    float eps) {
+    float eps, const void* __restrict__ y_bias) {
   constexpr bool EXACT = DT == LL_F32;
   __shared__ float red[4];
   const int64_t t = blockIdx.x;
@@ -135,6 +138,7 @@ __global__ __launch_bounds__(256) void gated_group_norm_cached_kernel(
       float s = 0.f;
       if (i < hi) {
         for (int p = 0; p < parts; ++p) s += ldv<DT>(y, (t * parts + p) * (int64_t)width + i);
+        if (y_bias) s += ldv<DT>(y_bias, i);
         if (shared) s += sscale * ldv<DT>(shared, t * (int64_t)width + i);
         if (gate) {
           float r = ldv<DT>(gate, t * gate_ld + i);
@@ -165,7 +169,7 @@ __global__ __launch_bounds__(256) void gated_group_norm_cached_kernel(
 #pragma unroll
       for (int k = 0; k < NV; ++k) {
         const int i = lo + tid + 256 * k;
-        if (i < hi) stv<DT>(h_out, t * (int64_t)width + i, val[k] * inv2 * ldv<DT>(next_w, i));
+        if (i < hi) stv<DT>(h_out, t * (int64_t)width + i, next_w ? val[k] * inv2 * ldv<DT>(next_w, i) : val[k]);
       }
     }
   }
@@ -201,7 +205,7 @@ __global__ __launch_bounds__(256) void gated_group_norm_vec_kernel(
     const float* x_in, float* x_out, void* __restrict__ h_out, const void* __restrict__ y, int parts,
     const void* __restrict__ shared, const float* __restrict__ shared_scale, const void* __restrict__ gate, int64_t gate_ld,
     const void* __restrict__ gate_bias, const void* __restrict__ post_w, const void* __restrict__ next_w, int width, int groups,
-    float eps) {
+    float eps, const void* __restrict__ y_bias) {
   constexpr bool EXACT = DT == LL_F32;
   __shared__ float red[4];
   const int64_t t = blockIdx.x;
@@ -220,6 +224,7 @@ __global__ __launch_bounds__(256) void gated_group_norm_vec_kernel(
       f32x4 s = {0.f, 0.f, 0.f, 0.f};
       if (i < hi) {
         for (int p = 0; p < parts; ++p) s += ld4<DT>(y, (t * parts + p) * (int64_t)width + i);
+        if (y_bias) s += ld4<DT>(y_bias, i);
         if (shared) s += sscale * ld4<DT>(shared, t * (int64_t)width + i);
         if (gate) {
           f32x4 r = ld4<DT>(gate, t * gate_ld + i);
@@ -257,10 +262,12 @@ __global__ __launch_bounds__(256) void gated_group_norm_vec_kernel(
       for (int k = 0; k < NV; ++k) {
         const int i = lo + 4 * (tid + 256 * k);
         if (i < hi) {
-          const f32x4 nw = ld4<DT>(next_w, i);
-          f32x4 o;
+          f32x4 o = val[k];   // (no next weight: the new residual itself, cast)
+          if (next_w) {
+            const f32x4 nw = ld4<DT>(next_w, i);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) o[e] = val[k][e] * inv2 * nw[e];
+            for (int e = 0; e < 4; ++e) o[e] = val[k][e] * inv2 * nw[e];
+          }
           st4<DT>(h_out, t * (int64_t)width + i, o);
         }
       }
@@ -352,14 +359,14 @@ __global__ __launch_bounds__(256) void softcap_kernel(void* __restrict__ x, int6
 extern "C" int ll_gated_group_norm(const float* x_in, float* x_out, void* h_out, const void* y, int64_t parts, const void* shared,
                                    const float* shared_scale, const void* gate, int64_t gate_ld, const void* gate_bias,
                                    const void* post_w, const void* next_w, int64_t n, int64_t width, int64_t groups, float eps,
-                                   int dtype, void* stream) {
+                                   const void* y_bias, int dtype, void* stream) {
   if (dtype != LL_F16 && dtype != LL_BF16 && dtype != LL_F32) return LL_ERR_DTYPE;
   if (n < 0 || width < 1 || width > (1 << 20) || groups < 1 || width % groups || parts < 0 || parts > 64) return LL_ERR_SHAPE;
   if (n == 0) return LL_OK;
   if (!x_in) return LL_ERR_ARG;
   if (y && (!x_out || !post_w || parts < 1)) return LL_ERR_ARG;
   if (!y && (!h_out || shared || gate)) return LL_ERR_ARG;
-  if (h_out && !next_w) return LL_ERR_ARG;
+  if (y_bias && !y) return LL_ERR_ARG;
   if (shared && !shared_scale) return LL_ERR_ARG;
   if (gate && gate_ld < width) return LL_ERR_SHAPE;
   if (!y) x_out = const_cast<float*>(x_in);
@@ -367,11 +374,12 @@ extern "C" int ll_gated_group_norm(const float* x_in, float* x_out, void* h_out,
   hipStream_t st = (hipStream_t)stream;
   const int64_t gs = width / groups;
 #define LL_GN_ARGS \
-  x_in, x_out, h_out, y, (int)parts, shared, shared_scale, gate, gate_ld, gate_bias, post_w, next_w, (int)width, (int)groups, eps
+  x_in, x_out, h_out, y, (int)parts, shared, shared_scale, gate, gate_ld, gate_bias, post_w, next_w, (int)width, (int)groups, eps, \
+  y_bias
   const int al = dtype == LL_F32 ? 16 : 8;   // bytes a four-channel piece of a storage-dtype row must be aligned to
   auto ok = [&](const void* p) { return !p || (reinterpret_cast<uintptr_t>(p) % al) == 0; };
   const bool vec = y && gs % 4 == 0 && gs <= 4096 && (!gate || gate_ld % 4 == 0) && ll_aligned16(x_in) && ll_aligned16(x_out) && ok(h_out) &&
-                   ok(y) && ok(shared) && ok(gate) && ok(gate_bias) && ok(post_w) && ok(next_w);
+                   ok(y) && ok(shared) && ok(gate) && ok(gate_bias) && ok(post_w) && ok(next_w) && ok(y_bias);
 #define CALL(DT)                                                                                          \
   if (vec && gs <= 1024) gated_group_norm_vec_kernel<DT, 1><<<grid, 256, 0, st>>>(LL_GN_ARGS);            \
   else if (vec && gs <= 2048) gated_group_norm_vec_kernel<DT, 2><<<grid, 256, 0, st>>>(LL_GN_ARGS);       \

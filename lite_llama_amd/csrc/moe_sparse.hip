@@ -31,6 +31,18 @@ __device__ __forceinline__ void stv(void* p, int64_t i, float v) {
 
 __device__ __forceinline__ float sigmoid_exact(float v) { return 1.0f / (1.0f + expf(-v)); }
 
+// the gated pair of an expert's first product.  limit < 0: silu(g) u; else the clamped form g' sigmoid(1.702 g') (u' + 1) with
+// g' = min(g, limit), u' = clamp(u, -limit, limit)
+template <int DT>
+__device__ __forceinline__ float glu_pair(float g, float u, float limit) {
+  if (limit >= 0.f) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit) + 1.0f;
+    return g * (DT == LL_F32 ? sigmoid_exact(1.702f * g) : ll_sigmoidf(1.702f * g)) * u;
+  }
+  return g * (DT == LL_F32 ? sigmoid_exact(g) : ll_sigmoidf(g)) * u;
+}
+
 // ------------------------------------------------------------------------------------------------------------------------
 // router, first launch: logits [n][experts (+ 1)] = h W^T in fp32.  A wave owns 8 tokens x 8 weight rows (x 2 rows for steps of
 // a few tokens, where more and shorter waves matter more than reuse) and walks the width
@@ -103,12 +115,16 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const void* __restri
 
 // router, second launch: one 64-thread workgroup per token over its logits.  LDS: scores [E], group score [G], group kept
 // [G], chosen scores [top].  SCORING 0: sigmoid scores, weights = chosen / sum; 1: the logits themselves rank the experts (no
-// groups) and the weights are the softmax over the chosen logits alone
-template <int SCORING>
+// groups) and the weights are the softmax over the chosen logits alone; 2: scores = softmax over ALL logits (no groups), the
+// experts are ranked by score + correction[e], the weights are the chosen scores themselves (not renormalised); the last
+// `identity` experts have no weights of their own -- a slot that chose one keeps its id (>= experts - identity, which the sort
+// by expert never places) and its score is added to extra_scale[t], the factor of the token's own input row
+template <int SCORING, int DT = LL_F32>
 __global__ __launch_bounds__(64) void group_select_kernel(const float* __restrict__ logits, int rows, int experts, int top,
                                                           int group_count, int group_keep, float route_scale,
                                                           int32_t* __restrict__ ids, float* __restrict__ weights,
-                                                          float* __restrict__ extra_scale) {
+                                                          float* __restrict__ extra_scale, const void* __restrict__ correction = nullptr,
+                                                          int identity = 0) {
   extern __shared__ float lds[];
   float* score = lds;                       // [experts]
   float* gscore = score + experts;          // [group_count]
@@ -116,6 +132,42 @@ __global__ __launch_bounds__(64) void group_select_kernel(const float* __restric
   float* chosen = gkeep + group_count;      // [top]
   const int64_t t = blockIdx.x;
   const int lane = threadIdx.x;
+  if constexpr (SCORING == 2) {
+    // softmax over all experts: every lane adds the exponentials in index order (one value for the whole wave); the ranking
+    // below sees score + correction, the weights the score alone
+    float top_z = -INFINITY;
+    for (int e = 0; e < experts; ++e) top_z = fmaxf(top_z, logits[t * rows + e]);
+    float total = 0.f;
+    for (int e = 0; e < experts; ++e) total += expf(logits[t * rows + e] - top_z);
+    float* plain = chosen + top;            // [experts] scores without the correction
+    for (int e = lane; e < experts; e += 64) {
+      const float sc = expf(logits[t * rows + e] - top_z) / total;
+      plain[e] = sc;
+      score[e] = correction ? sc + ldv<DT>(correction, e) : sc;
+    }
+    __syncthreads();
+    for (int e = lane; e < experts; e += 64) {
+      const float mine = score[e];
+      int rank = 0;
+      for (int o = 0; o < experts; ++o) {
+        const float sc = score[o];
+        rank += (sc > mine || (sc == mine && o < e)) ? 1 : 0;
+      }
+      if (rank < top) {
+        ids[t * top + rank] = e;
+        chosen[rank] = plain[e];
+        weights[t * top + rank] = plain[e] * route_scale;
+      }
+    }
+    __syncthreads();
+    if (extra_scale && lane == 0) {         // slots in rank order: the same sum whatever lane found which slot
+      float own = 0.f;
+      for (int k = 0; k < top; ++k)
+        if (ids[t * top + k] >= experts - identity) own += chosen[k];
+      extra_scale[t] = own * route_scale;
+    }
+    return;
+  }
   for (int e = lane; e < rows; e += 64) {
     const float z = logits[t * rows + e];
     if (e < experts) score[e] = SCORING == 1 ? z : sigmoid_exact(z);
@@ -218,7 +270,7 @@ __global__ __launch_bounds__(256) void moe_rows_gemm_kernel(const void* __restri
                                                             const float* __restrict__ slot_weight, void* __restrict__ out,
                                                             int64_t out_ld, const int32_t* __restrict__ sorted,
                                                             const int32_t* __restrict__ block_expert,
-                                                            const int32_t* __restrict__ num_post, int num_slots) {
+                                                            const int32_t* __restrict__ num_post, int num_slots, float glu_limit) {
   constexpr int BM = 32, BN = 64, BK = 32;
   __shared__ float As[BM][BK + 1];
   __shared__ int rows[BM];
@@ -264,8 +316,7 @@ __global__ __launch_bounds__(256) void moe_rows_gemm_kernel(const void* __restri
     if (slot >= num_slots) continue;
     float v;
     if (GLU) {
-      const float sg = DT == LL_F32 ? sigmoid_exact(acc_g[r]) : ll_sigmoidf(acc_g[r]);
-      v = acc_g[r] * sg * acc_u[r];
+      v = glu_pair<DT>(acc_g[r], acc_u[r], glu_limit);
     } else {
       v = slot_weight ? acc_g[r] * slot_weight[slot] : acc_g[r];
     }
@@ -296,7 +347,7 @@ __global__ __launch_bounds__(64) void moe_rows_gemm_mfma_kernel(const uint16_t* 
                                                                 const float* __restrict__ slot_weight, uint16_t* __restrict__ out,
                                                                 int64_t out_ld, const int32_t* __restrict__ sorted,
                                                                 const int32_t* __restrict__ block_expert,
-                                                                const int32_t* __restrict__ num_post, int num_slots) {
+                                                                const int32_t* __restrict__ num_post, int num_slots, float glu_limit) {
   constexpr int BM = 32, BN = 32;
   constexpr int NW = GLU ? 4 : 2;   // weight-row tiles of 16: gate 0..1, up 2..3
   const int block = blockIdx.x;
@@ -360,7 +411,7 @@ __global__ __launch_bounds__(64) void moe_rows_gemm_mfma_kernel(const uint16_t* 
         float v;
         if (GLU) {
           const float g = acc[j][m][r];
-          v = g * ll_sigmoidf(g) * acc[j + 2][m][r];
+          v = glu_pair<DT>(g, acc[j + 2][m][r], glu_limit);
         } else {
           v = acc[j][m][r] * sw;
         }
@@ -383,7 +434,7 @@ __global__ __launch_bounds__(256) void moe_rows_gemm_tiled_kernel(const uint16_t
                                                                   const float* __restrict__ slot_weight, uint16_t* __restrict__ out,
                                                                   int64_t out_ld, const int32_t* __restrict__ sorted,
                                                                   const int32_t* __restrict__ block_expert,
-                                                                  const int32_t* __restrict__ num_post, int num_slots) {
+                                                                  const int32_t* __restrict__ num_post, int num_slots, float glu_limit) {
   constexpr int BM = 128, WN = 128, BK = 64, STR = BK + 8, CW = GLU ? 64 : 128;
   __shared__ __attribute__((aligned(16))) uint16_t lds_a[BM * STR];
   __shared__ __attribute__((aligned(16))) uint16_t lds_w[WN * STR];
@@ -455,7 +506,7 @@ __global__ __launch_bounds__(256) void moe_rows_gemm_tiled_kernel(const uint16_t
       for (int r = 0; r < 4; ++r) {
         const int col = n0 + 16 * wave + 4 * c + r;
         const float g = acc[0][m][r];
-        if (col < N) orow[col] = from_f32<DT>(g * ll_sigmoidf(g) * acc[1][m][r]);
+        if (col < N) orow[col] = from_f32<DT>(glu_pair<DT>(g, acc[1][m][r], glu_limit));
       }
     } else {
       const float sw = slot_weight ? slot_weight[slot] : 1.0f;
@@ -482,11 +533,15 @@ __global__ __launch_bounds__(256) void moe_rows_gemm_tiled_kernel(const uint16_t
 // logits: fp32 scratch [n][experts + (w_extra ? 1 : 0)]
 extern "C" int ll_group_router(const void* h, int64_t h_ld, const void* w_router, const void* w_extra, int64_t n, int64_t width,
                                int64_t experts, int64_t top, int64_t group_count, int64_t group_keep, float route_scale, int scoring,
-                               int32_t* ids, float* weights, float* extra_scale, float* logits, int dtype, void* stream) {
+                               int32_t* ids, float* weights, float* extra_scale, float* logits, const void* correction, int64_t identity,
+                               int dtype, void* stream) {
   if (dtype != LL_F16 && dtype != LL_BF16 && dtype != LL_F32) return LL_ERR_DTYPE;
+  if (scoring == 2 && (group_count != 1 || w_extra || identity < 0 || identity > experts || (identity > 0 && !extra_scale)))
+    return LL_ERR_SHAPE;
+  if (scoring != 2 && (correction || identity)) return LL_ERR_SHAPE;
   if (n < 0 || width < 1 || h_ld < width || experts < 1 || experts > 4096 || top < 1 || top > experts || top > 64 || group_count < 1 ||
       experts % group_count || group_keep < 1 || group_keep > group_count || group_keep * (experts / group_count) < top ||
-      scoring < 0 || scoring > 1 || (scoring == 1 && group_count != 1))
+      scoring < 0 || scoring > 2 || (scoring == 1 && group_count != 1))
     return LL_ERR_SHAPE;
   if (n == 0) return LL_OK;
   if (!h || !w_router || !ids || !weights || !logits || (w_extra && !extra_scale)) return LL_ERR_ARG;
@@ -513,8 +568,14 @@ extern "C" int ll_group_router(const void* h, int64_t h_ld, const void* w_router
   }
 #undef LL_RL
 #undef LL_RL_ARGS
-  const size_t lds = sizeof(float) * (size_t)(experts + 2 * group_count + top);
-  if (scoring == 1)
+  const size_t lds = sizeof(float) * (size_t)(experts + 2 * group_count + top + (scoring == 2 ? experts : 0));
+  if (scoring == 2) {
+#define CALL(DT)                                                                                                                    \
+  group_select_kernel<2, DT><<<dim3((unsigned)n), 64, lds, st>>>(logits, rows, (int)experts, (int)top, 1, 1, route_scale, ids, weights, \
+                                                                 extra_scale, correction, (int)identity)
+    LL_BY_DTYPE(dtype, CALL);
+#undef CALL
+  } else if (scoring == 1)
     group_select_kernel<1><<<dim3((unsigned)n), 64, lds, st>>>(logits, rows, (int)experts, (int)top, (int)group_count, (int)group_keep,
                                                                route_scale, ids, weights, extra_scale);
   else
@@ -544,12 +605,14 @@ extern "C" int ll_moe_sort(const int32_t* ids, int64_t num_slots, int64_t expert
 }
 
 // glu != 0: w [experts][2 N][K] (gate rows, then up rows), out[slot][N] = silu(a_row Wg^T) * (a_row Wu^T) with a_row =
-// a[slot / a_div]; glu == 0: w [experts][N][K], out[slot][N] = (a[slot / a_div] W^T) * slot_weight[slot] (NULL: 1).
+// a[slot / a_div] (glu == 2: the clamped pair g' sigmoid(1.702 g') (u' + 1), g' = min(g, limit), u' = clamp(u, +-limit)); glu == 0: w [experts][N][K], out[slot][N] = (a[slot / a_div] W^T) * slot_weight[slot] (NULL: 1).
 extern "C" int ll_moe_rows_gemm(const void* a, int64_t a_ld, int64_t a_div, const void* w, int64_t w_stride_e, int64_t K, int64_t N,
                                 int glu, const float* slot_weight, void* out, int64_t out_ld, const int32_t* sorted,
                                 const int32_t* block_expert, const int32_t* num_post, int64_t num_slots, int64_t experts,
-                                int64_t block, int dtype, void* stream) {
+                                int64_t block, float limit, int dtype, void* stream) {
   if (dtype != LL_F16 && dtype != LL_BF16 && dtype != LL_F32) return LL_ERR_DTYPE;
+  if (glu < 0 || glu > 2 || (glu == 2 && !(limit >= 0.f))) return LL_ERR_SHAPE;
+  const float glu_limit = glu == 2 ? limit : -1.0f;
   if (num_slots < 0 || K < 1 || N < 1 || a_div < 1 || a_ld < K || out_ld < N || w_stride_e < (glu ? 2 : 1) * N * K || experts < 1 ||
       (block != 32 && block != 128))
     return LL_ERR_SHAPE;
@@ -565,7 +628,7 @@ extern "C" int ll_moe_rows_gemm(const void* a, int64_t a_ld, int64_t a_div, cons
 #define CALL_T(DT, G)                                                                                                          \
   moe_rows_gemm_tiled_kernel<DT, G><<<grid, 256, 0, st>>>((const uint16_t*)a, a_ld, (int)a_div, (const uint16_t*)w, w_stride_e, \
                                                           (int)K, (int)N, slot_weight, (uint16_t*)out, out_ld, sorted, block_expert, \
-                                                          num_post, (int)num_slots)
+                                                          num_post, (int)num_slots, glu_limit)
     if (dtype == LL_F16) { if (glu) CALL_T(LL_F16, true); else CALL_T(LL_F16, false); }
     else { if (glu) CALL_T(LL_BF16, true); else CALL_T(LL_BF16, false); }
 #undef CALL_T
@@ -576,7 +639,7 @@ extern "C" int ll_moe_rows_gemm(const void* a, int64_t a_ld, int64_t a_div, cons
 #define CALL_M(DT, G)                                                                                                         \
   moe_rows_gemm_mfma_kernel<DT, G><<<grid, 64, 0, st>>>((const uint16_t*)a, a_ld, (int)a_div, (const uint16_t*)w, w_stride_e, \
                                                         (int)K, (int)N, slot_weight, (uint16_t*)out, out_ld, sorted, block_expert, \
-                                                        num_post, (int)num_slots)
+                                                        num_post, (int)num_slots, glu_limit)
     if (dtype == LL_F16) { if (glu) CALL_M(LL_F16, true); else CALL_M(LL_F16, false); }
     else { if (glu) CALL_M(LL_BF16, true); else CALL_M(LL_BF16, false); }
 #undef CALL_M
@@ -585,9 +648,9 @@ extern "C" int ll_moe_rows_gemm(const void* a, int64_t a_ld, int64_t a_div, cons
   const dim3 grid((unsigned)max_blocks, (unsigned)((N + 63) / 64));
 #define CALL(DT)                                                                                                             \
   if (glu) moe_rows_gemm_kernel<DT, true><<<grid, 256, 0, st>>>(a, a_ld, (int)a_div, w, w_stride_e, (int)K, (int)N, slot_weight, \
-                                                                out, out_ld, sorted, block_expert, num_post, (int)num_slots);    \
+                                                                out, out_ld, sorted, block_expert, num_post, (int)num_slots, glu_limit);    \
   else moe_rows_gemm_kernel<DT, false><<<grid, 256, 0, st>>>(a, a_ld, (int)a_div, w, w_stride_e, (int)K, (int)N, slot_weight,   \
-                                                             out, out_ld, sorted, block_expert, num_post, (int)num_slots)
+                                                             out, out_ld, sorted, block_expert, num_post, (int)num_slots, glu_limit)
   LL_BY_DTYPE(dtype, CALL);
 #undef CALL
   return LL_LAUNCH_CHECK();

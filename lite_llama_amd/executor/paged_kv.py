@@ -109,8 +109,9 @@ class PagedStateCache(PagedKVPool):
                  previous_token: bool = False):
         """``runs``: one mapping per layer run: ``{"kind": "attention", "kv_heads", "dk", "dv"}``, ``{"kind": "latent", "rank",
         "rot"}`` or ``{"kind": "recurrent", "heads", "dk", "dv"}``, each with an optional ``"shift_width"``; attention runs may
-        add ``"conv_taps"`` / ``"conv_channels"`` (rows carried for a convolution of that many taps) and ``"value_mix": True``
-        (the first such run is the value source of the later ones).  ``previous_token``: keep each sequence's last token."""
+        add ``"conv_taps"`` / ``"conv_channels"`` (rows carried for a convolution of that many taps), ``"value_mix": True``
+        (the first such run is the value source of the later ones) and ``"state": (heads, dk, dv)`` (a recurrence that runs
+        beside the attention keeps its fp32 state in the same run).  ``previous_token``: keep each sequence's last token."""
         self.runs = [dict(r) for r in runs]
         self.dtype = dtype
         self.prev_token = torch.zeros(2, max_requests, dtype=torch.int32, device=device) if previous_token else None
@@ -133,7 +134,8 @@ class PagedStateCache(PagedKVPool):
             if r["kind"] == "attention":
                 buffers.append((torch.zeros(self.max_tokens, r["kv_heads"], r["dk"], dtype=dtype, device=dev),
                                 torch.zeros(self.max_tokens, r["kv_heads"], r["dv"], dtype=dtype, device=dev)))
-                self.recurrent.append(None)
+                # a mixer that runs a recurrence beside its attention keeps both: "state": (heads, dk, dv)
+                self.recurrent.append(torch.zeros(slots, *r["state"], dtype=torch.float32, device=dev) if r.get("state") else None)
             elif r["kind"] == "latent":
                 # one row [latent (rank) | rotated key part (rot)] per token: the keys of ONE key/value head; the values are the
                 # latent columns of the same rows (a row-strided view, nothing is stored twice)

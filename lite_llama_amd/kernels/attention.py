@@ -378,6 +378,36 @@ def conv_rope_cache(qkv, heads: int, kv_heads: int, dk: int, dv: int, step, k_ca
 
 
 @torch.no_grad()
+def rownorm_rope_cache(qkv, heads: int, kv_heads: int, dk: int, dv: int, step, k_cache, v_cache, *, q_weight=None, k_weight=None,
+                       eps: float = 0.0, freq=None, pairs: int = 0, value_scale: float = 1.0):
+    """Fused projection rows ``[q | k | v]`` -> queries ``[n, heads, dk]``; keys and values land in the cache rows
+    ``step.select``.  ``q_weight [heads dk]`` / ``k_weight [kv_heads dk]``: RMS norm over the WHOLE q (k) row -- one mean over
+    all heads' entries -- times a weight per entry (``None``: no norm).  Then entry ``i < pairs`` of every q / k head is rotated
+    with entry ``i + pairs`` by ``position * freq[i]``: ``(u, w) -> (u cos - w sin, w cos + u sin)``; entries from ``2 pairs`` on
+    pass unchanged.  Values enter the cache times ``value_scale`` (a constant factor of the attention's result, applied where
+    it costs nothing).  Norms, angles and the rotation are fp32."""
+    L.require_cuda(qkv, k_cache, v_cache, q_weight, k_weight, freq)
+    n, dt = qkv.shape[0], qkv.dtype
+    if qkv.dim() != 2 or qkv.stride(1) != 1 or qkv.shape[1] < (heads + kv_heads) * dk + kv_heads * dv or step.num_tokens != n:
+        raise ValueError("rownorm_rope_cache: rows hold [q | k | v] of the step's tokens")
+    if k_cache.dtype != dt or v_cache.dtype != dt or tuple(k_cache.shape[1:]) != (kv_heads, dk) \
+            or tuple(v_cache.shape[1:]) != (kv_heads, dv) or not (k_cache.is_contiguous() and v_cache.is_contiguous()):
+        raise ValueError("rownorm_rope_cache: caches are contiguous [rows, kv_heads, dk] / [rows, kv_heads, dv] in the rows' dtype")
+    for w, size in ((q_weight, heads * dk), (k_weight, kv_heads * dk)):
+        if w is not None and (w.dtype != dt or w.numel() != size or not w.is_contiguous()):
+            raise ValueError("rownorm_rope_cache: norm weights hold one entry per entry of the q / k row, in the rows' dtype")
+    if pairs and (freq is None or freq.dtype != torch.float32 or freq.numel() < pairs or not freq.is_contiguous() or 2 * pairs > dk):
+        raise ValueError("rownorm_rope_cache: fp32 frequencies, one per rotated pair of a head")
+    q = torch.empty(n, heads, dk, dtype=dt, device=qkv.device)
+    L.check(L.lib().ll_rownorm_rope_cache(qkv.data_ptr(), max(qkv.stride(0), qkv.shape[1]) if n <= 1 else qkv.stride(0), L.ptr(q_weight),
+                                          L.ptr(k_weight), float(eps), L.ptr(freq) if pairs else 0, int(pairs), float(value_scale),
+                                          step.tok_pos.data_ptr(), step.select.data_ptr(), q.data_ptr(), k_cache.data_ptr(),
+                                          v_cache.data_ptr(), n, heads, kv_heads, dk, dv, L.dtype_code(dt), L.stream_ptr()),
+            "rownorm_rope_cache")
+    return q
+
+
+@torch.no_grad()
 def ragged_attention(q, k_cache, v_cache, scale: float, step, token_table, sink=None, window: int = 0, keep_first: int = 0,
                      out=None):
     """Causal softmax attention of every token of a ragged step against positions ``0 .. its own`` of its sequence, keys and

@@ -251,14 +251,20 @@ def moe_router(x: torch.Tensor, gate_weight: torch.Tensor, top_k: int, norm_topk
 # ------------------------------------------------------------------------------------- #
 @torch.no_grad()
 def group_router(h: torch.Tensor, router_weight: torch.Tensor, top: int, group_count: int = 1, group_keep: int = 1,
-                 route_scale: float = 1.0, extra_weight: torch.Tensor | None = None, scoring: str = "sigmoid"):
+                 route_scale: float = 1.0, extra_weight: torch.Tensor | None = None, scoring: str = "sigmoid",
+                 correction: torch.Tensor | None = None, identity: int = 0):
     """``scores = sigmoid(router_weight h)`` in fp32 (``h`` in its storage dtype); the experts form ``group_count`` equal groups
     of neighbours, a group's score is the sum of its two best, the best ``group_keep`` groups stay eligible; the ``top`` best
     eligible experts are chosen.  Returns ``(ids int32 [n, top], weights fp32 [n, top], extra)``: weights = chosen scores /
     (their sum + 1e-20) * ``route_scale``, slot k = the k-th best; ``extra`` fp32 ``[n]`` = ``sigmoid(extra_weight . h)`` when a
     further weight row is given (the scale of a shared expert), else ``None``.  ``scoring="softmax_chosen"``: no sigmoid and no
-    groups -- the ``top`` largest logits are chosen and the weights are the softmax over the chosen logits alone."""
-    L.require_cuda(h, router_weight, extra_weight)
+    groups -- the ``top`` largest logits are chosen and the weights are the softmax over the chosen logits alone.
+    ``scoring="softmax_all"``: scores are the softmax over ALL router outputs; the experts are ranked by ``score +
+    correction[e]`` (``correction [experts]`` in the storage dtype, or ``None``) and weighted by their scores alone, not
+    renormalised.  The last ``identity`` router outputs stand for experts that return the token's own row: their slots keep
+    ids ``>= experts - identity`` (which :func:`sparse_glu_experts` leaves as zero rows) and ``extra`` is the sum of their
+    scores per token -- the factor of ``h`` itself in the sublayer's result."""
+    L.require_cuda(h, router_weight, extra_weight, correction)
     n, width = h.shape
     experts = router_weight.shape[0]
     if h.stride(1) != 1 or router_weight.dtype != h.dtype or not router_weight.is_contiguous() or router_weight.shape[1] != width:
@@ -267,23 +273,31 @@ def group_router(h: torch.Tensor, router_weight: torch.Tensor, top: int, group_c
         raise ValueError("group_router: the extra row has one weight per channel")
     ids = torch.empty(n, top, dtype=torch.int32, device=h.device)
     weights = torch.empty(n, top, dtype=torch.float32, device=h.device)
-    extra = torch.empty(n, dtype=torch.float32, device=h.device) if extra_weight is not None else None
+    if correction is not None and (correction.dtype != h.dtype or correction.numel() != experts or not correction.is_contiguous()):
+        raise ValueError("group_router: one correction per router output, in the rows' dtype")
+    if (correction is not None or identity) and scoring != "softmax_all":
+        raise ValueError("group_router: corrections and identity experts belong to the softmax_all scoring")
+    extra = torch.empty(n, dtype=torch.float32, device=h.device) if (extra_weight is not None or identity) else None
     logits = torch.empty(n, experts + (1 if extra_weight is not None else 0), dtype=torch.float32, device=h.device)
     L.check(L.lib().ll_group_router(h.data_ptr(), h.stride(0), router_weight.data_ptr(), L.ptr(extra_weight), n, width, experts,
                                     int(top), int(group_count), int(group_keep), float(route_scale),
-                                    {"sigmoid": 0, "softmax_chosen": 1}[scoring], ids.data_ptr(),
-                                    weights.data_ptr(), L.ptr(extra), logits.data_ptr(), L.dtype_code(h.dtype), L.stream_ptr()),
+                                    {"sigmoid": 0, "softmax_chosen": 1, "softmax_all": 2}[scoring], ids.data_ptr(),
+                                    weights.data_ptr(), L.ptr(extra), logits.data_ptr(), L.ptr(correction), int(identity),
+                                    L.dtype_code(h.dtype), L.stream_ptr()),
             "group_router")
     return ids, weights, extra
 
 
 @torch.no_grad()
 def sparse_glu_experts(h: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor, ids: torch.Tensor,
-                       weights: torch.Tensor) -> torch.Tensor:
+                       weights: torch.Tensor, *, limit: float | None = None, skipped_ids: bool = False) -> torch.Tensor:
     """Per slot (token, k): ``weights * down_e(silu(gate_e h) * up_e h)`` with ``e = ids[token, k]``; ``w_gate_up
     [experts, 2 ff, width]`` (gate rows, then up rows), ``w_down [experts, width, ff]``.  Returns the slots' rows
     ``[n, top, width]`` in the storage dtype (their sum over k is the caller's: the norm that follows adds them in fp32).
-    Slots are sorted by expert on the device; every product accumulates in fp32."""
+    Slots are sorted by expert on the device; every product accumulates in fp32.  ``limit``: the clamped pair
+    ``g' sigmoid(1.702 g') (u' + 1)`` with ``g' = min(gate, limit)``, ``u' = clamp(up, -limit, limit)`` instead of
+    ``silu(gate) up``.  ``skipped_ids``: some ids may lie beyond the experts (slots that no expert serves): their rows are
+    zeros."""
     L.require_cuda(h, w_gate_up, w_down, ids, weights)
     n, width = h.shape
     experts, two_ff, _ = w_gate_up.shape
@@ -305,12 +319,13 @@ def sparse_glu_experts(h: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.T
     L.check(lib.ll_moe_sort(ids.data_ptr(), slots, experts, block, counts.data_ptr(), sorted_ids.data_ptr(), block_expert.data_ptr(),
                             num_post.data_ptr(), L.stream_ptr()), "moe_sort")
     act = torch.empty(slots, ff, dtype=dt, device=h.device)
-    out = torch.empty(n, top, width, dtype=dt, device=h.device)
+    out = (torch.zeros if skipped_ids else torch.empty)(n, top, width, dtype=dt, device=h.device)
     code, st = L.dtype_code(dt), L.stream_ptr()
-    L.check(lib.ll_moe_rows_gemm(h.data_ptr(), h.stride(0), top, w_gate_up.data_ptr(), w_gate_up.stride(0), width, ff, 1, 0,
+    glu, lim = (1, 0.0) if limit is None else (2, float(limit))
+    L.check(lib.ll_moe_rows_gemm(h.data_ptr(), h.stride(0), top, w_gate_up.data_ptr(), w_gate_up.stride(0), width, ff, glu, 0,
                                  act.data_ptr(), ff, sorted_ids.data_ptr(), block_expert.data_ptr(), num_post.data_ptr(), slots,
-                                 experts, block, code, st), "moe_rows_gemm (gate|up)")
+                                 experts, block, lim, code, st), "moe_rows_gemm (gate|up)")
     L.check(lib.ll_moe_rows_gemm(act.data_ptr(), ff, 1, w_down.data_ptr(), w_down.stride(0), ff, width, 0, weights.data_ptr(),
                                  out.data_ptr(), width, sorted_ids.data_ptr(), block_expert.data_ptr(), num_post.data_ptr(), slots,
-                                 experts, block, code, st), "moe_rows_gemm (down)")
+                                 experts, block, 0.0, code, st), "moe_rows_gemm (down)")
     return out

@@ -487,34 +487,39 @@ class GatedUpdate:
     are summed: the experts a token chose), optionally ``+ shared_scale[t] * shared[t]``, times ``sigmoid(gate + gate_bias)``
     (``gate``: a column range of a projection's rows), to be normed with ``post_weight`` and added."""
 
-    __slots__ = ("y", "shared", "shared_scale", "gate", "gate_bias", "post_weight")
+    __slots__ = ("y", "shared", "shared_scale", "gate", "gate_bias", "post_weight", "bias")
 
-    def __init__(self, y, post_weight, gate=None, gate_bias=None, shared=None, shared_scale=None):
+    def __init__(self, y, post_weight, gate=None, gate_bias=None, shared=None, shared_scale=None, bias=None):
+        """``bias [width]``: added to the summed rows (the bias of the projection that produced them)."""
         self.y = y if y.dim() == 3 else y.unsqueeze(1)
         self.post_weight, self.gate, self.gate_bias, self.shared, self.shared_scale = post_weight, gate, gate_bias, shared, shared_scale
+        self.bias = bias
 
     def rows(self, index: torch.Tensor) -> "GatedUpdate":
         """The update of the listed tokens only."""
         pick = lambda t: None if t is None else t[index].contiguous()  # noqa: E731
-        return GatedUpdate(pick(self.y), self.post_weight, pick(self.gate), self.gate_bias, pick(self.shared), pick(self.shared_scale))
+        return GatedUpdate(pick(self.y), self.post_weight, pick(self.gate), self.gate_bias, pick(self.shared), pick(self.shared_scale),
+                           self.bias)
 
 
 @torch.no_grad()
-def gated_group_norm(x: torch.Tensor, update: "GatedUpdate | None", next_weight, eps: float, groups: int = 1):
+def gated_group_norm(x: torch.Tensor, update: "GatedUpdate | None", next_weight, eps: float, groups: int = 1, plain=None):
     """``x`` (fp32 residual ``[n, width]``, updated IN PLACE): ``x += groupnorm(update) * post_weight`` -- the update's rows
     summed, scaled by the sigmoid of its gate --, then ``h = groupnorm(x) * next_weight`` in the storage dtype
-    (``next_weight=None``: only the residual is updated).  ``groupnorm``: the row in ``groups`` equal consecutive parts, each
-    divided by ``sqrt(mean(part^2) + eps)``.  All sums, norms and the gate are fp32.  Returns ``h`` (or ``None``)."""
+    (``next_weight=None``: only the residual is updated; with ``plain`` = a storage dtype, ``h`` is the new residual itself in
+    that dtype: the next sublayer reads the stream without a norm in front).  ``groupnorm``: the row in ``groups`` equal
+    consecutive parts, each divided by ``sqrt(mean(part^2) + eps)``.  All sums, norms and the gate are fp32.  Returns ``h``
+    (or ``None``)."""
     L.require_cuda(x, next_weight)
     n, width = x.shape
     if x.dtype != torch.float32 or not x.is_contiguous() or width % groups:
         raise ValueError("gated_group_norm: a contiguous fp32 residual whose width the groups divide")
     u = update
-    dt = (next_weight if next_weight is not None else u.post_weight).dtype
-    h = torch.empty(n, width, dtype=dt, device=x.device) if next_weight is not None else None
+    dt = next_weight.dtype if next_weight is not None else plain if plain is not None else u.post_weight.dtype
+    h = torch.empty(n, width, dtype=dt, device=x.device) if (next_weight is not None or plain is not None) else None
     if next_weight is not None and (next_weight.numel() != width or not next_weight.is_contiguous()):
         raise ValueError("gated_group_norm: the norm weight has one entry per channel")
-    args = (0, 0, 0, 0, 0, 0, 0, 0)
+    args, y_bias = (0, 0, 0, 0, 0, 0, 0, 0), None
     if u is not None:
         if u.y.dtype != dt or u.y.shape[0] != n or u.y.shape[2] != width or not u.y.is_contiguous() or u.post_weight.dtype != dt:
             raise ValueError("gated_group_norm: the update is [n, parts, width] in the weights' dtype")
@@ -526,12 +531,15 @@ def gated_group_norm(x: torch.Tensor, update: "GatedUpdate | None", next_weight,
         if u.shared is not None and (u.shared.dtype != dt or u.shared.shape != (n, width) or not u.shared.is_contiguous()
                                      or u.shared_scale.dtype != torch.float32 or u.shared_scale.numel() != n):
             raise ValueError("gated_group_norm: the shared row is [n, width], its scale fp32 [n]")
+        y_bias = u.bias
+        if y_bias is not None and (y_bias.dtype != dt or y_bias.numel() != width or not y_bias.is_contiguous()):
+            raise ValueError("gated_group_norm: the update's bias has one entry per channel, in the weights' dtype")
         args = (u.y.data_ptr(), u.y.shape[1], L.ptr(u.shared), L.ptr(u.shared_scale), L.ptr(u.gate), gate_ld, L.ptr(u.gate_bias),
                 u.post_weight.data_ptr())
     elif h is None:
         return None
     L.check(L.lib().ll_gated_group_norm(x.data_ptr(), x.data_ptr(), L.ptr(h), *args, L.ptr(next_weight), n, width, int(groups),
-                                        float(eps), L.dtype_code(dt), L.stream_ptr()), "gated_group_norm")
+                                        float(eps), L.ptr(y_bias), L.dtype_code(dt), L.stream_ptr()), "gated_group_norm")
     return h
 
 

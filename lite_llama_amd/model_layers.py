@@ -21,14 +21,23 @@ description, out of mixers that take a ragged step (executor/ragged.py) and keep
                                0 in the denominator, values blended with those of the first such layer (kernels/attention.py)
   * :class:`ChosenSoftmaxMoE`  the largest router logits choose the experts, their weights are the softmax over the chosen
                                logits alone (kernels/fused_moe.py)
+  * :class:`WindowAttentionSSD`  two mixers side by side on one input: windowed softmax attention with whole-row q / k norms
+                               and a rotation of (i, i + dims / 2) pairs, and a state-space mixer (short convolution, scalar
+                               decay per head and token, gated grouped norm); one input and one output projection for both
+  * :class:`DecayLinearAttention`  linear attention with a fixed decay per head over silu features (kernels/recurrent.py)
+  * :class:`GatedLinearAttention`  linear attention with a decay per key entry from a low-rank projection
+  * :class:`BiasedGatedMLP`    ``down(silu(gate h + b) * (up h + b)) + b``
+  * :class:`CorrectedSoftmaxMoE`  softmax scores over all router outputs, experts chosen by score + correction and weighted by
+                               the score alone, clamped expert activations, router outputs that stand for "the input itself"
 
 The residual stream is fp32 throughout; every layer's residual add is fused into the norm that follows it
 (kernels/norm_act.py::add_rmsnorm_shift, which also applies the token shift in front of a mixer; or
 kernels/norm_act.py::gated_group_norm for layers that wrap each sublayer in two grouped norms and gate its result).
 Projections run through the framework's linear layers (library GEMM for unquantised weights), with everything that reads one
 input fused into one launch at load time.  Families: Rakevik (``"architecture": "Rakevik"``: :class:`MixerLayer`),
-Rukedra (:class:`SandwichLayer`) and Fekanex (:class:`ParallelLayer`: one norm per layer, mixer and feed-forward read its
-output side by side, and -- with a dense feed-forward -- share ONE input projection and ONE output projection).
+Rukedra (:class:`SandwichLayer`), Fekanex (:class:`ParallelLayer`: one norm per layer, mixer and feed-forward read its
+output side by side, and -- with a dense feed-forward -- share ONE input projection and ONE output projection) and Nivotar
+(:class:`PostNormLayer`: sublayers read the residual stream itself, the norm sits on each sublayer's result).
 """
 
 from __future__ import annotations
@@ -44,11 +53,12 @@ import torch.nn.functional as F
 
 from .distributed.parallel_state import get_tp_world_size
 from .kernels.activations import xielu
-from .kernels.attention import conv_rope_cache, latent_kv_prep, qk_norm_cache, ragged_attention, rotate_pairs, rotation_table
+from .kernels.attention import (conv_rope_cache, latent_kv_prep, qk_norm_cache, ragged_attention, rotate_pairs, rotation_table,
+                                rownorm_rope_cache)
 from .kernels.fused_moe import group_router, sparse_glu_experts
 from .kernels.norm_act import (GatedUpdate, SummedUpdate, add_rmsnorm_shift, cast_pair, embed_pair, gated_group_norm, glu_act,
                                residual_set, softcap_)
-from .kernels.recurrent import gated_linear_scan, mingru_scan
+from .kernels.recurrent import conv_act, gated_linear_scan, gated_out_norm, linear_scan, mingru_scan
 from .linear import ReplicatedLinear
 
 
@@ -94,8 +104,29 @@ class RotarySpec:
 
 
 @dataclass(frozen=True)
+class StateSpaceSpec:
+    """The state-space half of a two-branch mixer: ``heads`` heads of ``vdim`` channels over a state of ``state`` entries,
+    keys / queries shared by the heads of each of ``groups`` groups, a causal convolution of ``conv_taps`` taps in front, the
+    gated read-out normed in ``norm_groups`` equal parts."""
+    heads: int
+    vdim: int
+    state: int
+    groups: int
+    conv_taps: int
+    norm_groups: int
+
+    @property
+    def inner(self) -> int:
+        return self.heads * self.vdim
+
+    @property
+    def conv_channels(self) -> int:
+        return self.inner + 2 * self.groups * self.state
+
+
+@dataclass(frozen=True)
 class MixerSpec:
-    kind: str                   # "attention" | "hgrn2" | "latent_attention" | "mingru" | "conv_attention"
+    kind: str                   # "attention" | "hgrn2" | "latent_attention" | "mingru" | "conv_attention" | "attention_ssd" | "decay_linear" | "gla"
     heads: int = 1
     dim: int = 0                # per-head query / key width (latent attention: the unrotated part)
     vdim: int = 0               # per-head value width
@@ -116,15 +147,23 @@ class MixerSpec:
     out_gate: bool = False      # latent attention: heads times sigmoid(W_g h) before the output projection
     rotary: RotarySpec | None = None
     width: int = 0              # mingru: channels of the recurrence
+    ssd: StateSpaceSpec | None = None           # attention_ssd: the state-space branch beside the attention
+    branch_scales: tuple = (1.0, 1.0)           # attention_ssd: result = scales[0] * attention + scales[1] * state-space
+    decay: tuple = ()           # decay_linear: the fixed decay of every head
+    tau: float = 1.0            # gla: decay = sigmoid(.)^(1 / tau)
+    decay_rank: int = 0         # gla: width of the low-rank projection in front of the decay logits
 
 
 @dataclass(frozen=True)
 class MlpSpec:
     kind: str = "dense"         # "dense" | "moe"
     ff: int = 0                 # dense: hidden width; moe: hidden width of one expert
-    act: str = "xielu"          # dense: "xielu" (up / down) | "gelu_tanh" | "clamped" (gate / up / down)
+    act: str = "xielu"          # dense: "xielu" (up / down) | "gelu_tanh" | "clamped" | "silu" (gate / up / down)
     limit: float = 0.0          # "clamped": gate <= limit, |up| <= limit
     scoring: str = "sigmoid"    # moe: "sigmoid" (scores over groups) | "softmax_chosen" (largest logits, softmax over them)
+                                # | "softmax_all" (softmax over all outputs, chosen by score + correction)
+    identity: int = 0           # moe, "softmax_all": router outputs beyond `experts` that stand for the input itself
+    bias: bool = False          # dense: every projection carries a bias
     experts: int = 0
     top: int = 0
     group_count: int = 1
@@ -163,6 +202,7 @@ class LayeredGeometry:
     pair_mul_cur: int = 0
     logit_scale: float = 1.0    # logits = head(norm(x)) times this
     tied_head: bool = False     # the output head is the embedding table
+    post_norm: bool = False     # sublayers read the residual stream itself; each sublayer's RESULT is normed, then added
     extra: dict = field(default_factory=dict, compare=False)
 
     @property
@@ -180,7 +220,10 @@ class LayeredGeometry:
         return order + [(i, 0, False) for i in range(self.loop_stop, n)]
 
     @staticmethod
-    def from_config(config: Mapping, name: str = "rakevik") -> "LayeredGeometry":
+    def from_config(config: Mapping, name: str = "rakevik", shapes: Mapping | None = None) -> "LayeredGeometry":
+        """``shapes``: ``{tensor name: shape}`` of the checkpoint, for sizes that only a tensor's shape gives."""
+        if name == "nivotar":
+            return _nivotar_geometry(config, name, shapes or {})
         if name == "rukedra":
             return _rukedra_geometry(config, name)
         if name == "fekanex":
@@ -302,6 +345,63 @@ def _fekanex_geometry(config: Mapping, name: str) -> LayeredGeometry:
                            pair_buckets=int(pair.get("buckets") or 0), pair_mul_prev=int(pair.get("mul_prev") or 0),
                            pair_mul_cur=int(pair.get("mul_cur") or 0), logit_scale=float(config.get("logit_scale", 1.0)),
                            tied_head=True)
+
+
+def _nivotar_geometry(config: Mapping, name: str, shapes: Mapping) -> LayeredGeometry:
+    """Nivotar: per layer one of three mixers -- ``parallel`` (windowed attention with whole-row q / k norms and a half-split
+    rotation, beside a state-space mixer), ``lightning`` (linear attention with a fixed decay per head), ``gla`` (linear
+    attention with a decay per key entry) --, a dense biased silu feed-forward or experts chosen by a corrected softmax score
+    (some router outputs standing for the input itself), the norm on every sublayer's result, logits from the embedding
+    table.  The width of the low-rank projection in front of a ``gla`` layer's decay logits is the row count of its ``mix.a1``
+    tensor (``shapes``), or ``mixer.rank`` where a configuration is built without a checkpoint."""
+    layers = []
+    for index, entry in enumerate(config["layers"]):
+        m, kind = entry["mixer"], entry["type"]
+        if kind == "parallel":
+            a, r = m["left"], m["right"]
+            rot = RotarySpec(int(a["rot"]["dims"]), float(a["rot"]["base"])) if a.get("rot") else None
+            ssd = StateSpaceSpec(heads=int(r["heads"]), vdim=int(r["vdim"]), state=int(r["state"]), groups=int(r["groups"]),
+                                 conv_taps=int(r["conv"]), norm_groups=int(r["norm_groups"]))
+            spec = MixerSpec("attention_ssd", heads=int(a["heads"]), dim=int(a["dim"]), vdim=int(a["vdim"]),
+                             kv_heads=int(a.get("kv_heads") or a["heads"]), scale=float(a["scale"]), rotary=rot,
+                             window=int((a.get("mask") or {}).get("size") or 0), ssd=ssd,
+                             branch_scales=(float(m["left_scale"]), float(m["right_scale"])))
+            if spec.heads % spec.kv_heads:
+                raise ValueError(f"layer {index}: {spec.heads} query heads do not divide over {spec.kv_heads} key/value heads")
+            if rot is not None and (rot.dims > spec.dim or rot.dims % 2):
+                raise ValueError(f"layer {index}: {rot.dims} rotated entries do not fit heads of {spec.dim}")
+            if ssd.heads % ssd.groups or ssd.inner % ssd.norm_groups or ssd.conv_taps < 1:
+                raise ValueError(f"layer {index}: {ssd.heads} state-space heads of {ssd.vdim} do not divide over {ssd.groups} groups "
+                                 f"/ {ssd.norm_groups} norm parts")
+        elif kind == "lightning":
+            spec = MixerSpec("decay_linear", heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                             decay=tuple(float(d) for d in m["decay"]))
+            if len(spec.decay) != spec.heads:
+                raise ValueError(f"layer {index}: {len(spec.decay)} decays for {spec.heads} heads")
+        elif kind == "gla":
+            shape = shapes.get(f"l{index}.mix.a1")
+            rank = int(shape[0]) if shape is not None else int(m.get("rank") or 0)
+            spec = MixerSpec("gla", heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]), tau=float(m["tau"]), decay_rank=rank)
+            if not spec.tau > 0 or rank < 1:
+                raise ValueError(f"layer {index}: tau must be positive, and the decay projection's rank known (tensor mix.a1)")
+        else:
+            raise ValueError(f"unsupported mixer type {kind!r}; supported: parallel, lightning, gla")
+        mlp = entry.get("mlp")
+        if mlp is None:
+            mspec = None
+        elif mlp.get("kind", "dense") == "dense":
+            mspec = MlpSpec("dense", ff=int(mlp["ff"]), act="silu", bias=True)
+        elif mlp["kind"] == "moe":
+            r = mlp["router"]
+            mspec = MlpSpec("moe", ff=int(mlp["expert"]["ff"]), act="clamped", limit=float(mlp["expert"]["limit"]),
+                            experts=int(r["experts"]), top=int(r["top"]), scoring="softmax_all", identity=int(r.get("identity") or 0))
+            if not 1 <= mspec.top <= mspec.experts + mspec.identity or mspec.experts < 1 or mspec.limit < 0:
+                raise ValueError(f"layer {index}: {mspec.top} of {mspec.experts} + {mspec.identity} experts cannot be chosen")
+        else:
+            raise ValueError(f"unsupported feed-forward kind {mlp.get('kind')!r}; supported: dense, moe")
+        layers.append(LayerSpec(spec, ff=mspec.ff if mspec else 0, mlp_kind=mspec.kind if mspec else "dense", mlp=mspec))
+    return LayeredGeometry(name=name, vocab_size=int(config["vocab"]), width=int(config["width"]), eps=float(config["norm"]["eps"]),
+                           layers=tuple(layers), token_shift=False, tied_head=True, post_norm=True)
 
 
 def _linear(inp: int, out: int) -> ReplicatedLinear:
@@ -603,8 +703,157 @@ class ChosenSoftmaxMoE(nn.Module):
         return sparse_glu_experts(h, self.gate_up_weight, self.down_weight, ids, weights)
 
 
+class WindowAttentionSSD(nn.Module):
+    """Two mixers side by side on the same input, ``a_l * attention(h) + a_r * ssd(h)``, with ONE input projection
+    ``q | k | v | z | u B C | dt`` and ONE output projection ``[W_o,left | W_o,right]`` over ``[a_l * heads' outputs | a_r *
+    gated, normed read-out]``, whose fp32 accumulation is the sum of the branches.  Attention: q and k RMS-normed over their
+    whole rows, rotated in (i, i + dims / 2) pairs, a sliding window over the paged cache (``a_l`` rides on the cached values).
+    State-space branch: ``u B C`` through a causal convolution and silu, then per head ``S <- exp(-exp(A_log) dt) S + dt B u^T``,
+    ``y = S^T C + D u`` (B, C shared by the heads of a group), ``y silu(z)`` RMS-normed in equal parts."""
+
+    def __init__(self, width: int, spec: MixerSpec, eps: float):
+        super().__init__()
+        self.spec, self.eps = spec, eps
+        s, r = spec, spec.ssd
+        self.qkv = (s.heads + s.kv_heads) * s.dim + s.kv_heads * s.vdim
+        self.z_off = self.qkv
+        self.conv_off = self.z_off + r.inner
+        self.dt_off = self.conv_off + r.conv_channels
+        self.in_proj = _linear(width, self.dt_off + r.heads)
+        self.q_norm_weight = _vector(s.heads * s.dim)
+        self.k_norm_weight = _vector(s.kv_heads * s.dim)
+        self.conv_weight = nn.Parameter(torch.zeros(r.conv_channels, r.conv_taps, dtype=torch.float16), requires_grad=False)
+        self.conv_bias = _vector(r.conv_channels)
+        self.dt_bias, self.a_log, self.skip = _vector(r.heads), _vector(r.heads), _vector(r.heads)
+        self.ssd_norm_weight = _vector(r.inner)
+        self.heads_width = s.heads * s.vdim
+        self.out_proj = _linear(self.heads_width + r.inner, width)
+        self._freq_values = s.rotary.table()[0] if s.rotary is not None else []
+        self.pairs = len(self._freq_values)
+        self._freq = None   # fp32 on the device of the first step (not a buffer: a module-wide cast must not touch the angles)
+
+    def cache_run(self) -> dict:
+        s, r = self.spec, self.spec.ssd
+        return {"kind": "attention", "kv_heads": s.kv_heads, "dk": s.dim, "dv": s.vdim, "state": (r.heads, r.state, r.vdim),
+                "conv_taps": r.conv_taps, "conv_channels": r.conv_channels}
+
+    def forward(self, h, step, cache, run: int, token_table):
+        s, r = self.spec, self.spec.ssd
+        rows = self.in_proj(h)
+        if self.pairs and (self._freq is None or self._freq.device != h.device):
+            self._freq = torch.tensor(self._freq_values, dtype=torch.float64).to(torch.float32).to(h.device)
+        mixed = torch.empty(h.shape[0], self.heads_width + r.inner, dtype=h.dtype, device=h.device)
+        k_cache, v_cache = cache.kv_buffer[run]
+        q = rownorm_rope_cache(rows, s.heads, s.kv_heads, s.dim, s.vdim, step, k_cache, v_cache, q_weight=self.q_norm_weight,
+                               k_weight=self.k_norm_weight, eps=self.eps, freq=self._freq, pairs=self.pairs,
+                               value_scale=s.branch_scales[0])
+        ragged_attention(q, k_cache, v_cache, s.scale, step, token_table, window=s.window, out=mixed[:, :self.heads_width])
+        ubc = conv_act(rows[:, self.conv_off:self.dt_off], self.conv_weight, self.conv_bias, step, cache.conv[run])
+        gn = r.groups * r.state
+        o = linear_scan(ubc[:, r.inner + gn:], ubc[:, r.inner:r.inner + gn], ubc[:, :r.inner], r.heads, r.state, r.vdim, step,
+                        cache.recurrent[run], qk_heads=r.groups, dt=rows[:, self.dt_off:], dt_bias=self.dt_bias, a_log=self.a_log,
+                        skip=self.skip)
+        gated_out_norm(o, self.ssd_norm_weight, self.eps, parts=r.norm_groups, gate=rows[:, self.z_off:self.conv_off],
+                       gate_kind="silu", gate_first=True, scale=s.branch_scales[1], out=mixed[:, self.heads_width:])
+        return self.out_proj(mixed)
+
+
+class DecayLinearAttention(nn.Module):
+    """``q | k | v | g`` in one projection; per head ``S <- decay_h S + silu(k) silu(v)^T``, ``o = S^T silu(q)`` over the fp32
+    state slots; the heads side by side RMS-normed together, times ``sigmoid(g)``; output projection."""
+
+    def __init__(self, width: int, spec: MixerSpec, eps: float):
+        super().__init__()
+        self.spec, self.eps = spec, eps
+        self.qk, self.v = spec.heads * spec.dim, spec.heads * spec.vdim
+        self.in_proj = _linear(width, 2 * self.qk + 2 * self.v)
+        self.out_norm_weight = _vector(self.v)
+        self.o_proj = _linear(self.v, width)
+        self._decay = None   # fp32 on the device of the first step (not a buffer: a module-wide cast must not round the decays)
+
+    def cache_run(self) -> dict:
+        return {"kind": "recurrent", "heads": self.spec.heads, "dk": self.spec.dim, "dv": self.spec.vdim}
+
+    def forward(self, h, step, cache, run: int, token_table):
+        s, qk, v = self.spec, self.qk, self.v
+        rows = self.in_proj(h)
+        if self._decay is None or self._decay.device != h.device:
+            self._decay = torch.tensor(s.decay, dtype=torch.float64).to(torch.float32).to(h.device)
+        o = linear_scan(rows[:, :qk], rows[:, qk:2 * qk], rows[:, 2 * qk:2 * qk + v], s.heads, s.dim, s.vdim, step,
+                        cache.recurrent[run], act=True, head_decay=self._decay)
+        return self.o_proj(gated_out_norm(o, self.out_norm_weight, self.eps, gate=rows[:, 2 * qk + v:], gate_kind="sigmoid"))
+
+
+class GatedLinearAttention(nn.Module):
+    """``q | k | v | g | a`` in one projection (``a``: the low-rank input of the decay logits); per head
+    ``S <- diag(alpha) S + k v^T``, ``o = S^T q / sqrt(dim)`` with ``alpha = sigmoid(W_a2 a + b)^(1 / tau)`` per key entry;
+    every head RMS-normed with one shared weight, times ``silu(g)``; output projection."""
+
+    def __init__(self, width: int, spec: MixerSpec, eps: float):
+        super().__init__()
+        self.spec, self.eps = spec, eps
+        rank = spec.decay_rank
+        self.qk, self.v = spec.heads * spec.dim, spec.heads * spec.vdim
+        self.in_proj = _linear(width, 2 * self.qk + 2 * self.v + rank)
+        self.decay_proj = _linear(rank, self.qk)
+        self.decay_bias = _vector(self.qk)
+        self.out_norm_weight = _vector(spec.vdim)
+        self.o_proj = _linear(self.v, width)
+
+    def cache_run(self) -> dict:
+        return {"kind": "recurrent", "heads": self.spec.heads, "dk": self.spec.dim, "dv": self.spec.vdim}
+
+    def forward(self, h, step, cache, run: int, token_table):
+        s, qk, v = self.spec, self.qk, self.v
+        rows = self.in_proj(h)
+        logits = self.decay_proj(rows[:, 2 * qk + 2 * v:].contiguous())
+        o = linear_scan(rows[:, :qk], rows[:, qk:2 * qk], rows[:, 2 * qk:2 * qk + v], s.heads, s.dim, s.vdim, step,
+                        cache.recurrent[run], q_scale=s.dim ** -0.5, gate=logits, gate_bias=self.decay_bias, tau=s.tau)
+        return self.o_proj(gated_out_norm(o, self.out_norm_weight, self.eps, parts=s.heads, gate=rows[:, 2 * qk + v:2 * qk + 2 * v],
+                                          gate_kind="silu"))
+
+
+class BiasedGatedMLP(nn.Module):
+    """``down(silu(gate h + b_g) * (up h + b_u)) + b_d``; ``gate | up`` are one projection.  The down projection's bias is
+    not added here: it rides with the result into the norm launch that follows."""
+
+    def __init__(self, width: int, ff: int):
+        super().__init__()
+        self.ff = ff
+        self.in_proj = ReplicatedLinear(width, 2 * ff, bias=True)
+        self.down_proj = _linear(ff, width)
+        self.down_bias = _vector(width)
+
+    def forward(self, h):
+        return self.down_proj(glu_act(self.in_proj(h), self.ff, "silu")), self.down_bias, None, None
+
+
+class CorrectedSoftmaxMoE(nn.Module):
+    """Scores are the softmax (fp32) over ALL router outputs; the ``top`` largest ``score + correction`` choose, the scores
+    alone weigh (not renormalised).  Experts are clamped gated feed-forwards without biases, run as grouped products over slots
+    sorted by expert.  The last ``identity`` router outputs have no weights: a token that chooses one gets its own input row
+    times the score.  Neither the slots' rows nor that row are summed here: they ride into the norm launch that follows."""
+
+    def __init__(self, width: int, spec: MlpSpec):
+        super().__init__()
+        self.spec = spec
+        outputs = spec.experts + spec.identity
+        self.router_weight = nn.Parameter(torch.zeros(outputs, width, dtype=torch.float16), requires_grad=False)
+        self.correction = _vector(outputs)
+        self.gate_up_weight = nn.Parameter(torch.zeros(spec.experts, 2 * spec.ff, width, dtype=torch.float16), requires_grad=False)
+        self.down_weight = nn.Parameter(torch.zeros(spec.experts, width, spec.ff, dtype=torch.float16), requires_grad=False)
+
+    def forward(self, h):
+        s = self.spec
+        ids, weights, own = group_router(h, self.router_weight, s.top, scoring=s.scoring, correction=self.correction,
+                                         identity=s.identity)
+        y = sparse_glu_experts(h, self.gate_up_weight, self.down_weight, ids, weights, limit=s.limit, skipped_ids=s.identity > 0)
+        return y, None, (h if s.identity else None), own
+
+
 MIXERS = {"attention": SinkAttention, "hgrn2": GatedLinearMixer, "latent_attention": LatentAttention, "mingru": MinGRU,
-          "conv_attention": ConvRotaryAttention}
+          "conv_attention": ConvRotaryAttention, "attention_ssd": WindowAttentionSSD, "decay_linear": DecayLinearAttention,
+          "gla": GatedLinearAttention}
 
 
 class MixerLayer(nn.Module):
@@ -690,6 +939,34 @@ class ParallelLayer(nn.Module):
         return x, SummedUpdate(row, self.experts(h) if self.experts is not None else None)
 
 
+class PostNormLayer(nn.Module):
+    """``x <- x + norm_1(mixer(x))``, then ``x <- x + norm_2(feed_forward(x))``: sublayers read the residual stream itself (cast
+    to the storage dtype), the norm sits on each sublayer's RESULT.  A result is carried as a :class:`GatedUpdate` into the
+    launch that opens the next sublayer: norm of the result, residual add and the cast of the new stream are one launch."""
+
+    def __init__(self, geo: LayeredGeometry, spec: LayerSpec):
+        super().__init__()
+        self.eps = geo.eps
+        w, m = geo.width, spec.mixer
+        self.norm1_weight = _vector(w)
+        self.mixer = MIXERS[m.kind](w, m, geo.eps)
+        self.mlp = None
+        if spec.mlp is not None:
+            self.norm2_weight = _vector(w)
+            self.mlp = CorrectedSoftmaxMoE(w, spec.mlp) if spec.mlp.kind == "moe" else BiasedGatedMLP(w, spec.mlp.ff)
+
+    def forward(self, x, pending, step, cache, run: int, token_table):
+        """``(x, pending)``: the fp32 residual (updated in place) and the update still to enter it.  Returns the same pair."""
+        dt = self.norm1_weight.dtype
+        h = gated_group_norm(x, pending, None, self.eps, plain=dt)
+        pending = GatedUpdate(self.mixer(h, step, cache, run, token_table), self.norm1_weight)
+        if self.mlp is not None:
+            h = gated_group_norm(x, pending, None, self.eps, plain=dt)
+            y, bias, own, own_scale = self.mlp(h)
+            pending = GatedUpdate(y, self.norm2_weight, shared=own, shared_scale=own_scale, bias=bias)
+        return x, pending
+
+
 # ------------------------------------------------------------------------------------- #
 # the model
 # ------------------------------------------------------------------------------------- #
@@ -703,7 +980,7 @@ class LayeredLM(nn.Module):
         self.geo = geo
         self.embed_tokens = nn.Embedding(geo.vocab_size, geo.width, dtype=torch.float16)
         self.embed_tokens.weight.requires_grad_(False)
-        make = SandwichLayer if geo.sandwich else ParallelLayer if geo.parallel else MixerLayer
+        make = SandwichLayer if geo.sandwich else ParallelLayer if geo.parallel else PostNormLayer if geo.post_norm else MixerLayer
         # a layer that borrows weights IS the other layer's module (which may come later in the stack); its cache run stays its own
         built = [make(geo, spec) if spec.weights_of is None else None for spec in geo.layers]
         self.layers = nn.ModuleList(built[i] if spec.weights_of is None else built[spec.weights_of] for i, spec in enumerate(geo.layers))
@@ -752,7 +1029,7 @@ class LayeredLM(nn.Module):
                 x, delta = residual_set(y, self.loop_step[pass_no]), None
             x, delta = self.layers[index](x, delta, step, cache, run, token_table)
             if collect_layers is not None:
-                if self.geo.sandwich:   # (diagnostics: the pending update is applied to a copy)
+                if self.geo.sandwich or self.geo.post_norm:   # (diagnostics: the pending update is applied to a copy)
                     seen = x.clone()
                     gated_group_norm(seen, delta, None, self.geo.eps, self.geo.norm_groups)
                     collect_layers.append(seen)
@@ -763,7 +1040,7 @@ class LayeredLM(nn.Module):
         if logits_rows is None:
             return None
         x = x[logits_rows].contiguous()
-        if self.geo.sandwich:
+        if self.geo.sandwich or self.geo.post_norm:
             h = gated_group_norm(x, delta.rows(logits_rows) if delta is not None else None, self.norm_weight, self.geo.eps,
                                  self.geo.norm_groups)
         else:
@@ -798,12 +1075,17 @@ class LayeredLM(nn.Module):
             elif name in ("embed_tokens.weight", "pair_table"):
                 fill(p, std=1.0)
             elif leaf in ("norm1_weight", "norm2_weight", "norm_weight", "q_norm_weight", "k_norm_weight", "out_norm_weight",
-                          "norm1b_weight", "norm2b_weight", "kv_norm_weight"):
+                          "norm1b_weight", "norm2b_weight", "kv_norm_weight", "ssd_norm_weight"):
                 fill(p, std=0.1, mean=1.0)
             elif leaf in ("uk_weight", "uv_weight", "router_weight", "gate_up_weight", "down_weight", "shared_scale_weight"):
                 fill(p, std=1.0 / (p.shape[-1] ** 0.5))
-            elif leaf in ("rg1_bias", "rg2_bias", "z_bias", "x_bias", "qkv_bias"):
+            elif leaf in ("rg1_bias", "rg2_bias", "z_bias", "x_bias", "qkv_bias", "conv_bias", "down_bias", "decay_bias", "dt_bias") \
+                    or name.endswith("proj.bias"):
                 fill(p, std=0.5)
+            elif leaf in ("a_log", "skip"):
+                fill(p, lo=-1.0, hi=1.0)
+            elif leaf == "correction":
+                fill(p, std=0.02)
             elif leaf == "conv_weight":
                 fill(p, std=p.shape[1] ** -0.5)
             elif leaf == "value_blend":

@@ -707,19 +707,101 @@ def _fekanex_translator(geo) -> Translator:
     return translate
 
 
+def _nivotar_translator(geo) -> Translator:
+    """Tensor names of a Nivotar checkpoint -> parameters of :class:`lite_llama_amd.model_layers.LayeredLM` built from
+    :class:`PostNormLayer`.  Everything that reads a mixer's input lands in its row range of the mixer's ONE input projection
+    (``left.q | left.k | left.v | right.in`` -- itself ``z | u B C | dt`` --; ``q | k | v | g``; ``q | k | v | g | a1``); the two
+    branches' ``left.o`` / ``right.o`` in their COLUMN ranges of one output projection; ``mlp.gate / up`` (and their biases)
+    in the halves of one projection; experts ``mlp.e<k>.*`` in the stacked expert tensors.  The output head is the embedding
+    table (no tensor of its own)."""
+    fixed = {"embed": "embed_tokens.weight", "final.norm": "norm_weight"}
+    plain = {"norm1": "norm1_weight", "norm2": "norm2_weight", "mix.o": "mixer.o_proj.weight", "mix.norm": "mixer.out_norm_weight",
+             "mix.a2": "mixer.decay_proj.weight", "mix.a2.b": "mixer.decay_bias", "mix.left.q.norm": "mixer.q_norm_weight",
+             "mix.left.k.norm": "mixer.k_norm_weight", "mix.right.conv": "mixer.conv_weight", "mix.right.conv.b": "mixer.conv_bias",
+             "mix.right.dt_bias": "mixer.dt_bias", "mix.right.A_log": "mixer.a_log", "mix.right.D": "mixer.skip",
+             "mix.right.norm": "mixer.ssd_norm_weight", "mlp.down": "mlp.down_proj.weight", "mlp.down.b": "mlp.down_bias",
+             "mlp.router": "mlp.router_weight", "mlp.correction": "mlp.correction"}
+    expert_leaf = re.compile(r"^mlp\.e(\d+)\.(gate|up|down)$")
+
+    def fused(spec):
+        """``{checkpoint leaf: (parameter, Region)}`` of one layer."""
+        m, out = spec.mixer, {}
+
+        def rows(param, members):
+            at = 0
+            for leaf, count in members:
+                out[leaf] = (param, Region(rows=(at, count)))
+                at += count
+            return at
+
+        if m.kind == "attention_ssd":
+            r = m.ssd
+            rows("mixer.in_proj.weight", (("mix.left.q", m.heads * m.dim), ("mix.left.k", m.kv_heads * m.dim),
+                                          ("mix.left.v", m.kv_heads * m.vdim), ("mix.right.in", 2 * r.inner + 2 * r.groups * r.state + r.heads)))
+            out["mix.left.o"] = ("mixer.out_proj.weight", Region(cols=(0, m.heads * m.vdim)))
+            out["mix.right.o"] = ("mixer.out_proj.weight", Region(cols=(m.heads * m.vdim, r.inner)))
+        else:
+            qk, v = m.heads * m.dim, m.heads * m.vdim
+            rows("mixer.in_proj.weight", (("mix.q", qk), ("mix.k", qk), ("mix.v", v), ("mix.g", v))
+                 + ((("mix.a1", m.decay_rank),) if m.kind == "gla" else ()))
+        if spec.mlp is not None and spec.mlp.kind == "dense":
+            ff = spec.mlp.ff
+            rows("mlp.in_proj.weight", (("mlp.gate", ff), ("mlp.up", ff)))
+            rows("mlp.in_proj.bias", (("mlp.gate.b", ff), ("mlp.up.b", ff)))
+        return out
+
+    members = [fused(spec) for spec in geo.layers]
+
+    def translate(key: str) -> Target:
+        if key in fixed:
+            return fixed[key], whole
+        m = re.match(r"^l(\d+)\.(.+)$", key)
+        if m is None or int(m.group(1)) >= len(geo.layers):
+            return key, whole  # unknown: load_weights reports it
+        index, leaf = int(m.group(1)), m.group(2)
+        if leaf in members[index]:
+            name, region = members[index][leaf]
+            return f"layers.{index}.{name}", region
+        e = expert_leaf.match(leaf)
+        if e is not None:
+            k, proj = int(e.group(1)), e.group(2)
+            if proj == "down":
+                return f"layers.{index}.mlp.down_weight", expert(k)
+            return f"layers.{index}.mlp.gate_up_weight", expert_half(k, 0 if proj == "gate" else 1)
+        return f"layers.{index}.{plain.get(leaf, leaf)}", whole
+
+    return translate
+
+
+def tensor_shapes(checkpoints_dir: str | Path) -> dict[str, tuple[int, ...]]:
+    """``{tensor name: shape}`` of a directory's safetensors files (headers only: no tensor is read)."""
+    from safetensors import safe_open
+
+    shapes = {}
+    for path in hf_weight_files(checkpoints_dir):
+        if path.suffix != ".safetensors":
+            continue
+        with safe_open(path, framework="pt", device="cpu") as shard:
+            for key in shard.keys():
+                shapes[key] = tuple(shard.get_slice(key).get_shape())
+    return shapes
+
+
 def _load_layered(config: Mapping, checkpoints_dir, device, dtype=None, **_):
     from .model_layers import LayeredGeometry, LayeredLM
 
-    geo = LayeredGeometry.from_config(config, name=model_family(config))
+    family = model_family(config)
+    geo = LayeredGeometry.from_config(config, name=family, shapes=tensor_shapes(checkpoints_dir) if family == "nivotar" else None)
     model = LayeredLM(geo, dtype=dtype or torch.bfloat16).to(device)
     translator = (_rukedra_translator(geo) if geo.sandwich else _fekanex_translator(geo) if geo.parallel
-                  else _layered_translator(geo))
+                  else _nivotar_translator(geo) if geo.post_norm else _layered_translator(geo))
     with torch.no_grad():
         load_weights(model, hf_weights_iterator(checkpoints_dir, device), translator)
     return model.eval()
 
 
-MODEL_FAMILIES: dict[str, Callable] = {"rakevik": _load_layered, "rukedra": _load_layered, "fekanex": _load_layered}
+MODEL_FAMILIES: dict[str, Callable] = {"rakevik": _load_layered, "rukedra": _load_layered, "fekanex": _load_layered,
+                                       "nivotar": _load_layered}
 
 
 def load_pretrained(checkpoints_dir: str | Path, *, device: str | torch.device = "cuda", quantization: str | None = None,
