@@ -107,6 +107,19 @@ def causal_conv(u, w, b):
     return y
 
 
+def decay_scan(q, k, v, a):
+    """One head, token by token: S <- diag(a_t) S + k_t v_t^T, o_t = S^T q_t.  ``q, k [T, d]``, ``v [T, dv]``, ``a [T, d]`` (or
+    anything that broadcasts to it: ``[T, 1]``, a number).  Returns ``(o [T, dv], the last S)``."""
+    T, d = k.shape
+    a = torch.as_tensor(a, dtype=q.dtype) * torch.ones(T, d, dtype=q.dtype)
+    S = torch.zeros(d, v.shape[1], dtype=q.dtype)
+    o = torch.zeros(T, v.shape[1], dtype=q.dtype)
+    for i in range(T):
+        S = a[i][:, None] * S + torch.outer(k[i], v[i])
+        o[i] = S.T @ q[i]
+    return o, S
+
+
 def ssd(x, t, p, m, eps):
     T, dt_ = x.shape[0], x.dtype
     H, dv, N, G = int(m["heads"]), int(m["vdim"]), int(m["state"]), int(m["groups"])
@@ -123,10 +136,8 @@ def ssd(x, t, p, m, eps):
     y = torch.zeros(T, H, dv, dtype=dt_)
     for h in range(H):
         g = h // (H // G)
-        S = torch.zeros(N, dv, dtype=dt_)
-        for i in range(T):
-            S = torch.exp(-rate[h] * dt[i, h]) * S + dt[i, h] * torch.outer(B[i, g], u[i, h])
-            y[i, h] = S.T @ C[i, g] + D[h] * u[i, h]
+        o, _ = decay_scan(C[:, g], B[:, g], dt[:, h, None] * u[:, h], torch.exp(-rate[h] * dt[:, h, None]))
+        y[:, h] = o + D[h] * u[:, h]
     y = y.view(T, inner) * silu(z)
     parts = int(m["norm_groups"])
     y = rms_norm(y.view(T, parts, inner // parts), None, eps).view(T, inner) * t[p + "norm"].to(dt_)
@@ -149,10 +160,7 @@ def lightning(x, t, p, m, eps):
     v = silu(x @ t[p + "v"].to(dt).T).view(T, H, dv)
     o = torch.zeros(T, H, dv, dtype=dt)
     for h in range(H):
-        S = torch.zeros(d, dv, dtype=dt)
-        for i in range(T):
-            S = float(m["decay"][h]) * S + torch.outer(k[i, h], v[i, h])
-            o[i, h] = S.T @ q[i, h]
+        o[:, h], _ = decay_scan(q[:, h], k[:, h], v[:, h], float(m["decay"][h]))
     o = rms_norm(o.view(T, H * dv), t[p + "norm"].to(dt), eps) * torch.sigmoid(x @ t[p + "g"].to(dt).T)
     return o @ t[p + "o"].to(dt).T
 
@@ -167,10 +175,7 @@ def gla(x, t, p, m, eps):
     alpha = torch.exp(torch.nn.functional.logsigmoid(zed) / float(m["tau"])).view(T, H, d)
     o = torch.zeros(T, H, dv, dtype=dt)
     for h in range(H):
-        S = torch.zeros(d, dv, dtype=dt)
-        for i in range(T):
-            S = alpha[i, h][:, None] * S + torch.outer(k[i, h], v[i, h])
-            o[i, h] = S.T @ q[i, h]
+        o[:, h], _ = decay_scan(q[:, h], k[:, h], v[:, h], alpha[:, h])
     o = rms_norm(o, t[p + "norm"].to(dt), eps).view(T, H * dv) * silu(x @ t[p + "g"].to(dt).T)
     return o @ t[p + "o"].to(dt).T
 
