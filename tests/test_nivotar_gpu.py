@@ -119,7 +119,7 @@ def test_a_value_written_far_back_is_read_hundreds_of_tokens_later_through_many_
     rows[far, dk:2 * dk] = 0.0
     rows[far, dk + 3] = 4.0
     rows[far, 2 * dk:] = bf(torch.linspace(-8, 8, dv))
-    for probe in (600 + far // 2, 699):
+    for probe in (600 + far // 4, 699):
         rows[probe, :dk] = 0.0
         rows[probe, 3] = 2.0
     state = torch.randn(2, 1, dk, dv, device=DEV)
