@@ -106,6 +106,13 @@ def parse():
                          "--layered-dtype picks the dtype")
     ap.add_argument("--fekanex-sizes", default="compact,wide", help="which size points of benchmarks/fekanex_bench.py::SIZES to run")
     ap.add_argument("--fekanex-model-only", action="store_true", help="skip the per-kernel table (a short run for a kernel trace)")
+    ap.add_argument("--nivotar", action="store_true",
+                    help="instead of the headline: prefill / decode throughput and per-kernel roofline fractions of the Nivotar design "
+                         "(windowed attention beside a state-space mixer, linear attention with fixed and per-entry decays, corrected "
+                         "softmax experts, norms on the sublayers' results) beside the closest model of the layered family "
+                         "(benchmarks/nivotar_bench.py); --layered-dtype picks the dtype")
+    ap.add_argument("--nivotar-sizes", default="compact,wide", help="which size points of benchmarks/nivotar_bench.py::SIZES to run")
+    ap.add_argument("--nivotar-model-only", action="store_true", help="skip the per-kernel table (a short run for a kernel trace)")
     ap.add_argument("--rukedra-sizes", default="compact,wide", help="which size points of benchmarks/rukedra_bench.py::SIZES to run")
     ap.add_argument("--rukedra-model-only", action="store_true", help="skip the per-kernel table (a short run for a kernel trace)")
     ap.add_argument("--no-reference-order", action="store_true",
@@ -941,6 +948,11 @@ def main():
         from benchmarks.rukedra_bench import run as rukedra_run
 
         print(json.dumps(rukedra_run(args.layered_dtype, sizes=tuple(args.rukedra_sizes.split(",")), kernels=not args.rukedra_model_only)))
+        return
+    if args.nivotar:
+        from benchmarks.nivotar_bench import run as nivotar_run
+
+        print(json.dumps(nivotar_run(args.layered_dtype, sizes=tuple(args.nivotar_sizes.split(",")), kernels=not args.nivotar_model_only)))
         return
     if args.fekanex:
         from benchmarks.fekanex_bench import run as fekanex_run
