@@ -220,7 +220,7 @@ SIZES = {
                     experts=32, identity=2, top=4, eff=704),
     # a wider model: 24 query heads on 8 key/value heads with values of 96, 48 state-space heads, more and smaller experts
     "wide": dict(width=3072, heads=24, kv_heads=8, dim=128, vdim=96, rot=128, window=1024, ssd_heads=48, ssd_vdim=64, state=64, groups=8,
-                 taps=4, parts=8, lin_heads=24, lin_dim=64, lin_vdim=128, gla_heads=12, gla_dim=256, gla_vdim=256, rank=32, ff=8192,
+                 taps=4, parts=8, lin_heads=24, lin_dim=64, lin_vdim=128, gla_heads=12, gla_dim=128, gla_vdim=256, rank=32, ff=8192,
                  experts=64, identity=4, top=8, eff=512),
 }
 
