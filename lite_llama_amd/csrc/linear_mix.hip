@@ -298,6 +298,205 @@ __global__ __launch_bounds__(256) void rownorm_rope_cache_kernel(
   for (int i = tid; i < vn; i += 256) stv<DT>(v_cache, row * vn + i, ldv<DT>(rows, at + qn + kn + i) * value_scale);
 }
 
+// eight consecutive storage-dtype values at element i (a multiple of 8 from a 16-byte aligned base) as fp32
+template <int DT>
+__device__ __forceinline__ void ld8(const void* p, int64_t i, float (&o)[8]) {
+  if constexpr (DT == LL_F32) {
+    const f32x4 a = *reinterpret_cast<const f32x4*>((const float*)p + i), b = *reinterpret_cast<const f32x4*>((const float*)p + i + 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { o[e] = a[e]; o[4 + e] = b[e]; }
+  } else {
+    const U16x8 u = *reinterpret_cast<const U16x8*>((const uint16_t*)p + i);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = to_f32<DT>(u.v[e]);
+  }
+}
+template <int DT>
+__device__ __forceinline__ void st8(void* p, int64_t i, const float (&o)[8]) {
+  if constexpr (DT == LL_F32) {
+    *reinterpret_cast<f32x4*>((float*)p + i) = f32x4{o[0], o[1], o[2], o[3]};
+    *reinterpret_cast<f32x4*>((float*)p + i + 4) = f32x4{o[4], o[5], o[6], o[7]};
+  } else {
+    U16x8 u;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) u.v[e] = from_f32<DT>(o[e]);
+    *reinterpret_cast<U16x8*>((uint16_t*)p + i) = u;
+  }
+}
+
+// The read-out norm for long parts: one workgroup per (token, part), same arithmetic per element as the wave form.
+template <int DT>
+__global__ __launch_bounds__(256) void gated_out_norm_block_kernel(void* __restrict__ out, int64_t out_ld, const float* __restrict__ o,
+                                                                   const void* __restrict__ gate, int64_t gate_ld, int gate_kind,
+                                                                   int gate_first, const void* __restrict__ w, int w_len, float eps,
+                                                                   float out_scale, int parts, int ps) {
+  __shared__ float red[4];
+  const int64_t item = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int64_t t = item / parts;
+  const int c0 = (int)(item - t * parts) * ps;
+  const float* src = o + t * (int64_t)parts * ps + c0;
+  auto gate_at = [&](int cc) -> float {
+    const float g = ldv<DT>(gate, t * gate_ld + c0 + cc);
+    const float s = act_sigmoid<DT>(g);
+    return gate_kind == 1 ? g * s : s;
+  };
+  float ss = 0.f;
+  for (int cc = tid; cc < ps; cc += 256) {
+    float v = src[cc];
+    if (gate_kind && gate_first) v *= gate_at(cc);
+    ss += v * v;
+  }
+  ss = block_sum256(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)ps + eps);
+  for (int cc = tid; cc < ps; cc += 256) {
+    float v = src[cc];
+    const float g = gate_kind ? gate_at(cc) : 1.0f;
+    if (gate_first) v *= g;
+    v = v * inv * (w ? ldv<DT>(w, (c0 + cc) % w_len) : 1.0f);
+    if (!gate_first) v *= g;
+    stv<DT>(out, t * out_ld + c0 + cc, v * out_scale);
+  }
+}
+
+// The convolution in 16-byte pieces: a thread owns eight consecutive channels of one token; the taps' weights of those
+// channels are one contiguous run of 8 TAPS values.  Same sums in the same order as the plain form.
+template <int DT, int TAPS>
+__global__ __launch_bounds__(256) void conv_act_vec_kernel(void* __restrict__ out, int64_t out_ld, const void* __restrict__ rows, int64_t ld,
+                                                           const void* __restrict__ w, const void* __restrict__ bias, int channels,
+                                                           void* __restrict__ state, int64_t state_half, const int32_t* __restrict__ tok_seq,
+                                                           const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ seq_start,
+                                                           const int32_t* __restrict__ seq_first_pos, const int32_t* __restrict__ seq_slot,
+                                                           const int32_t* __restrict__ seq_parity, int64_t pieces) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= pieces) return;
+  const int per = channels >> 3;
+  const int64_t t = idx / per;
+  const int c = (int)(idx - t * per) << 3;
+  const int seq = tok_seq[t], pos = tok_pos[t];
+  const int start = seq_start[seq], first = seq_first_pos[seq];
+  const int64_t slot_at = (int64_t)seq_slot[seq] * (TAPS - 1) * channels;
+  const int par = seq_parity[seq] & 1;
+  const int64_t in_at = par * state_half + slot_at, out_at = (par ^ 1) * state_half + slot_at;
+  auto raw_at = [&](int p, float (&u)[8]) {
+    if (p >= first) ld8<DT>(rows, (int64_t)(start + (p - first)) * ld + c, u);
+    else ld8<DT>(state, in_at + (int64_t)(p - first + TAPS - 1) * channels + c, u);
+  };
+  float wl[8 * TAPS];
+#pragma unroll
+  for (int j = 0; j < TAPS; ++j) {
+    float piece[8];
+    ld8<DT>(w, (int64_t)c * TAPS + 8 * j, piece);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) wl[8 * j + e] = piece[e];
+  }
+  float acc[8];
+  if (bias) ld8<DT>(bias, c, acc);
+  else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+  }
+#pragma unroll
+  for (int j = 0; j < TAPS; ++j) {
+    const int p = pos - (TAPS - 1 - j);
+    if (p < 0) continue;
+    float u[8];
+    raw_at(p, u);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] += wl[e * TAPS + j] * u[e];
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = acc[e] * act_sigmoid<DT>(acc[e]);
+  st8<DT>(out, t * out_ld + c, acc);
+  if (TAPS > 1 && t == seq_start[seq + 1] - 1) {
+#pragma unroll
+    for (int s = 0; s < TAPS - 1; ++s) {
+      const int p = pos + 1 - (TAPS - 1) + s;
+      float u[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      if (p >= 0) raw_at(p, u);
+      st8<DT>(state, out_at + (int64_t)s * channels + c, u);
+    }
+  }
+}
+
+// The whole-row norms and the rotation in 16-byte pieces (head widths, rotated halves and row strides multiples of 8): a
+// thread sums the squares of its pieces, then -- after the two workgroup sums -- reads each piece again with the piece it is
+// rotated with.  Same arithmetic per entry as the plain form; the sums of squares are taken in piece order.
+template <int DT>
+__global__ __launch_bounds__(256) void rownorm_rope_cache_vec_kernel(
+    const void* __restrict__ rows, int64_t ld, const void* __restrict__ q_w, const void* __restrict__ k_w, float eps,
+    const float* __restrict__ freq, int half, float value_scale, const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ select,
+    void* __restrict__ q_out, void* __restrict__ k_cache, void* __restrict__ v_cache, int heads, int kv_heads, int dk, int dv) {
+  extern __shared__ float cs[];   // [half] cos, [half] sin
+  __shared__ float red[4];
+  const int64_t t = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int qn = heads * dk, kn = kv_heads * dk, vn = kv_heads * dv;
+  const int64_t at = t * ld;
+  const float pos = (float)tok_pos[t];
+  for (int i = tid; i < half; i += 256) {
+    float s, c;
+    sincosf(pos * freq[i], &s, &c);
+    cs[i] = c;
+    cs[half + i] = s;
+  }
+  float sq = 0.f, sk = 0.f;
+  for (int i = tid * 8; i < qn + kn; i += 2048) {
+    float u[8];
+    ld8<DT>(rows, at + i, u);
+    float s = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s += u[e] * u[e];
+    if (i < qn) sq += s;
+    else sk += s;
+  }
+  sq = block_sum256(sq, red);
+  sk = block_sum256(sk, red);   // (its first barrier also publishes cs)
+  const float inv_q = q_w ? 1.0f / sqrtf(sq / (float)qn + eps) : 1.0f;
+  const float inv_k = k_w ? 1.0f / sqrtf(sk / (float)kn + eps) : 1.0f;
+  const int64_t row = select[t];
+  for (int i = tid * 8; i < qn + kn; i += 2048) {
+    const bool is_q = i < qn;
+    const int idx = is_q ? i : i - qn;                 // entry inside the q (k) row
+    const int64_t base = is_q ? at : at + qn;
+    const void* w = is_q ? q_w : k_w;
+    const float inv = is_q ? inv_q : inv_k;
+    float v[8];
+    ld8<DT>(rows, base + idx, v);
+    if (w) {
+      float wv[8];
+      ld8<DT>(w, idx, wv);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = v[e] * inv * wv[e];
+    }
+    const int in_head = idx % dk;
+    if (in_head < 2 * half) {
+      const bool low = in_head < half;
+      const int other = low ? idx + half : idx - half;
+      const int a0 = low ? in_head : in_head - half;   // first angle of the piece
+      float p[8];
+      ld8<DT>(rows, base + other, p);
+      if (w) {
+        float wv[8];
+        ld8<DT>(w, other, wv);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) p[e] = p[e] * inv * wv[e];
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = low ? v[e] * cs[a0 + e] - p[e] * cs[half + a0 + e] : v[e] * cs[a0 + e] + p[e] * cs[half + a0 + e];
+    }
+    if (is_q) st8<DT>(q_out, t * qn + idx, v);
+    else st8<DT>(k_cache, row * kn + idx, v);
+  }
+  for (int i = tid * 8; i < vn; i += 2048) {
+    float v[8];
+    ld8<DT>(rows, at + qn + kn + i, v);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] *= value_scale;
+    st8<DT>(v_cache, row * vn + i, v);
+  }
+}
+
 }  // namespace
 
 #define LL_BY_DTYPE(dtype, CALL)                  \
@@ -361,7 +560,15 @@ extern "C" int ll_gated_out_norm(void* out, int64_t out_ld, const float* o, cons
   if (n == 0) return LL_OK;
   if (!out || !o || (gate_kind && (!gate || gate_ld < width))) return LL_ERR_ARG;
   const int64_t items = n * parts;
-  if ((items + 3) / 4 > 0x7fffffffll) return LL_ERR_SHAPE;
+  if (items > 0x7fffffffll) return LL_ERR_SHAPE;
+  if (width / parts >= 512) {   // long parts: a workgroup each (the form depends on the part's length only)
+#define CALL(DT)                                                                                                                   \
+  gated_out_norm_block_kernel<DT><<<dim3((unsigned)items), 256, 0, (hipStream_t)stream>>>(                                         \
+      out, out_ld, o, gate, gate_ld, gate_kind, gate_first ? 1 : 0, w, (int)(w ? w_len : 1), eps, out_scale, (int)parts, (int)(width / parts))
+    LL_BY_DTYPE(dtype, CALL);
+#undef CALL
+    return LL_LAUNCH_CHECK();
+  }
 #define CALL(DT)                                                                                                                 \
   gated_out_norm_kernel<DT><<<dim3((unsigned)((items + 3) / 4)), 256, 0, (hipStream_t)stream>>>(                                 \
       out, out_ld, o, gate, gate_ld, gate_kind, gate_first ? 1 : 0, w, (int)(w ? w_len : 1), eps, out_scale, items, (int)parts, \
@@ -381,6 +588,25 @@ extern "C" int ll_conv_act(void* out, int64_t out_ld, const void* rows, int64_t 
   if (n == 0) return LL_OK;
   if (!out || !rows || !w || !tok_seq || !tok_pos || !seq_start || !seq_first_pos || !seq_slot || !seq_parity || (taps > 1 && !state))
     return LL_ERR_ARG;
+  const int al = dtype == LL_F32 ? 4 : 8;   // elements per 16 bytes
+  if (taps <= 4 && channels % 8 == 0 && ld % al == 0 && out_ld % al == 0 && ll_aligned16(rows) && ll_aligned16(out) && ll_aligned16(w) &&
+      (!bias || ll_aligned16(bias)) && (taps == 1 || ll_aligned16(state)) ) {
+    // (fp32 pieces of eight are two 16-byte accesses: strides that are multiples of 4 keep both aligned)
+    const int64_t pieces = n * (channels / 8);
+    const dim3 vgrid((unsigned)((pieces + 255) / 256));
+#define CALL_T(DT, T)                                                                                                                \
+  conv_act_vec_kernel<DT, T><<<vgrid, 256, 0, (hipStream_t)stream>>>(out, out_ld, rows, ld, w, bias, (int)channels, state, state_half, \
+                                                                     tok_seq, tok_pos, seq_start, seq_first_pos, seq_slot, seq_parity, pieces)
+#define CALL(DT)                      \
+  if (taps == 1) CALL_T(DT, 1);       \
+  else if (taps == 2) CALL_T(DT, 2);  \
+  else if (taps == 3) CALL_T(DT, 3);  \
+  else CALL_T(DT, 4)
+    LL_BY_DTYPE(dtype, CALL);
+#undef CALL
+#undef CALL_T
+    return LL_LAUNCH_CHECK();
+  }
   const dim3 grid((unsigned)n, (unsigned)((channels + 255) / 256));
 #define CALL(DT)                                                                                                                     \
   conv_act_kernel<DT><<<grid, 256, 0, (hipStream_t)stream>>>(out, out_ld, rows, ld, w, bias, (int)channels, (int)taps, state, state_half, \
@@ -401,6 +627,17 @@ extern "C" int ll_rownorm_rope_cache(const void* rows, int64_t ld, const void* q
   if (n == 0) return LL_OK;
   if (!rows || !tok_pos || !select || !q_out || !k_cache || !v_cache || (pairs && !freq)) return LL_ERR_ARG;
   const size_t lds = sizeof(float) * (size_t)(2 * pairs + 1);
+  const int al = dtype == LL_F32 ? 4 : 8;
+  if (dk % 8 == 0 && dv % 8 == 0 && pairs % 8 == 0 && ld % al == 0 && ll_aligned16(rows) && ll_aligned16(q_out) && ll_aligned16(k_cache) &&
+      ll_aligned16(v_cache) && (!q_w || ll_aligned16(q_w)) && (!k_w || ll_aligned16(k_w))) {
+#define CALL(DT)                                                                                                                 \
+  rownorm_rope_cache_vec_kernel<DT><<<dim3((unsigned)n), 256, lds, (hipStream_t)stream>>>(                                       \
+      rows, ld, q_w, k_w, eps, freq, (int)pairs, value_scale, tok_pos, select, q_out, k_cache, v_cache, (int)heads, (int)kv_heads, \
+      (int)dk, (int)dv)
+    LL_BY_DTYPE(dtype, CALL);
+#undef CALL
+    return LL_LAUNCH_CHECK();
+  }
 #define CALL(DT)                                                                                                                 \
   rownorm_rope_cache_kernel<DT><<<dim3((unsigned)n), 256, lds, (hipStream_t)stream>>>(                                           \
       rows, ld, q_w, k_w, eps, freq, (int)pairs, value_scale, tok_pos, select, q_out, k_cache, v_cache, (int)heads, (int)kv_heads, \
