@@ -57,6 +57,8 @@ __device__ __forceinline__ float act_sigmoid(float v) {
 // ln(sigmoid(z)) without cancellation on either side
 __device__ __forceinline__ float log_sigmoid(float z) { return z >= 0.f ? -log1pf(expf(-z)) : z - log1pf(expf(z)); }
 __device__ __forceinline__ float softplus(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+// sigmoid(z)^(1 / tau): ONE definition for the scan and for the pass that evaluates a step's decays ahead of it
+__device__ __forceinline__ float entry_decay(float z, float inv_tau) { return expf(log_sigmoid(z) * inv_tau); }
 
 struct ScanArgs {
   const void* q;   // [n, q_ld]: head j's entries at columns j dk ..
@@ -72,6 +74,7 @@ struct ScanArgs {
   int64_t gate_ld;
   const void* gate_bias;
   float inv_tau;
+  const float* decay_pre;    // kind 1: the decays of this step [n, heads dk], evaluated ahead of the scan (or NULL: evaluated here)
   const void* dt;            // kind 2: rows [n, dt_ld] of one raw step size per head; dt_bias, a_log, skip: [heads]
   int64_t dt_ld;
   const void* dt_bias;
@@ -84,6 +87,18 @@ struct ScanArgs {
   const int32_t* seq_slot;
   float* state;              // fp32 [slots, heads, dk, dv]
 };
+
+// The decays of a step's tokens per key entry, once per token: the scan's dv / 16 column workgroups of a head would each evaluate
+// them again (two exponentials and a logarithm per entry), which for runs of many tokens costs more than the walk over the state.
+template <int DT>
+__global__ __launch_bounds__(256) void entry_decay_kernel(float* __restrict__ out, const void* __restrict__ gate, int64_t gate_ld,
+                                                          const void* __restrict__ gate_bias, float inv_tau, int64_t total, int cols) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const int64_t t = i / cols;
+  const int c = (int)(i - t * cols);
+  out[i] = entry_decay(ldv<DT>(gate, t * gate_ld + c) + ldv<DT>(gate_bias, c), inv_tau);
+}
 
 // One workgroup per (sequence of the step, head, 16 columns of the state).  Thread (kg, col): column col of the slice, state
 // rows kg, kg + 16, ... in registers.  Tokens are taken tb at a time: decay, key and query of every key entry are staged in
@@ -134,7 +149,8 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(const ScanArgs a) {
       float dec;
       if (kind == 0) dec = a.head_decay[head];
       else if (kind == 1)
-        dec = expf(log_sigmoid(ldv<DT>(a.gate, row * a.gate_ld + head * dk + kk) + ldv<DT>(a.gate_bias, head * dk + kk)) * a.inv_tau);
+        dec = a.decay_pre ? a.decay_pre[(row * heads + head) * dk + kk]
+                          : entry_decay(ldv<DT>(a.gate, row * a.gate_ld + head * dk + kk) + ldv<DT>(a.gate_bias, head * dk + kk), a.inv_tau);
       else dec = sd[2 * tt];
       sg[i] = f32x4{dec, kv, qv * a.q_scale, 0.f};
     }
@@ -513,7 +529,7 @@ extern "C" int ll_linear_scan(const void* q, int64_t q_ld, const void* k, int64_
                               const void* gate, int64_t gate_ld, const void* gate_bias, float inv_tau, const void* dt, int64_t dt_ld,
                               const void* dt_bias, const void* a_log, const void* skip, float* o, int64_t batch,
                               const int32_t* seq_start, const int32_t* seq_first_pos, const int32_t* seq_slot, float* state,
-                              int dtype, void* stream) {
+                              float* decay_scratch, int64_t n, int dtype, void* stream) {
   if (dtype != LL_F16 && dtype != LL_BF16 && dtype != LL_F32) return LL_ERR_DTYPE;
   if (batch < 0 || heads < 1 || heads > 65535 || !ll_linear_scan_supported(dk, dv) || qk_rep < 1 || heads % qk_rep || kind < 0 ||
       kind > 2 || (dv + 15) / 16 > 65535)
@@ -529,12 +545,22 @@ extern "C" int ll_linear_scan(const void* q, int64_t q_ld, const void* k, int64_
   a.q = q; a.k = k; a.v = v; a.q_ld = q_ld; a.k_ld = k_ld; a.v_ld = v_ld;
   a.heads = (int)heads; a.dk = (int)dk; a.dv = (int)dv; a.qk_rep = (int)qk_rep; a.kind = kind; a.act = act; a.q_scale = q_scale;
   a.head_decay = head_decay; a.gate = gate; a.gate_ld = gate_ld; a.gate_bias = gate_bias; a.inv_tau = inv_tau;
+  a.decay_pre = nullptr;
   a.dt = dt; a.dt_ld = dt_ld; a.dt_bias = dt_bias; a.a_log = a_log; a.skip = skip; a.o = o;
   a.tb = dk <= 128 ? 16 : 8;
   a.seq_start = seq_start; a.seq_first_pos = seq_first_pos; a.seq_slot = seq_slot; a.state = state;
   const size_t lds = sizeof(float) * (size_t)(a.tb * (4 * dk + 16 + 16 + 256 + 2));
   const dim3 grid((unsigned)batch, (unsigned)heads, (unsigned)((dv + 15) / 16));
   hipStream_t st = (hipStream_t)stream;
+  if (kind == 1 && decay_scratch && n > 0) {   // decays once per token and entry, ahead of the scan: fp32 [n, heads dk]
+    const int64_t total = n * heads * dk;
+    if ((total + 255) / 256 > 0x7fffffffll) return LL_ERR_SHAPE;
+#define CALL(DT) \
+  entry_decay_kernel<DT><<<dim3((unsigned)((total + 255) / 256)), 256, 0, st>>>(decay_scratch, gate, gate_ld, gate_bias, inv_tau, total, (int)(heads * dk))
+    LL_BY_DTYPE(dtype, CALL);
+#undef CALL
+    a.decay_pre = decay_scratch;
+  }
   const int rmax = (int)((dk + 15) / 16);
 #define CALL_W(DT, R, E) linear_scan_kernel<DT, R, E><<<grid, 256, lds, st>>>(a)
 #define CALL(DT)                                \

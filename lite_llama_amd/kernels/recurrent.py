@@ -147,12 +147,15 @@ def linear_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, heads: int, d
         if dt.dtype != st or dt.shape[0] != n:
             raise ValueError("linear_scan: step sizes in the rows' dtype, one row per token")
     o = torch.empty(n, heads * dv, dtype=torch.float32, device=q.device)
+    # runs of several tokens: the decays per key entry are evaluated once per token ahead of the scan (its column workgroups
+    # would each evaluate them again); decode steps evaluate them in the scan
+    pre = torch.empty(n, heads * dk, dtype=torch.float32, device=q.device) if (kind == 1 and step.longest_run != 1 and dv > 16) else None
     L.check(L.lib().ll_linear_scan(
         q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0), heads, dk, dv, heads // qk_heads, kind,
         1 if act else 0, float(q_scale), L.ptr(head_decay), L.ptr(gate), gate.stride(0) if gate is not None else 0, L.ptr(gate_bias),
         1.0 / float(tau), L.ptr(dt), dt.stride(0) if dt is not None else 0, L.ptr(dt_bias), L.ptr(a_log), L.ptr(skip), o.data_ptr(),
         step.num_seqs, step.seq_start.data_ptr(), step.seq_first_pos.data_ptr(), step.seq_slot.data_ptr(), state.data_ptr(),
-        L.dtype_code(st), L.stream_ptr()), "linear_scan")
+        L.ptr(pre), n, L.dtype_code(st), L.stream_ptr()), "linear_scan")
     return o
 
 

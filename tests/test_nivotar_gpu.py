@@ -106,6 +106,28 @@ def test_decaying_state_over_portions_of_every_size_and_stale_slots(dtype, kind,
         _close(got[s], want.view(-1, vw), 3e-5 if dtype == torch.float32 else 2e-2)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_decays_evaluated_ahead_of_the_scan_are_the_ones_evaluated_inside_it(dtype):
+    """Runs of several tokens evaluate the per-entry decays in a pass of their own, decoded tokens inside the scan: the same
+    bits, so a prompt in one portion and token by token leaves the same state."""
+    from lite_llama_amd.kernels.recurrent import linear_scan
+
+    g = torch.Generator().manual_seed(11)
+    heads, dk, dv, n = 2, 24, 40, 37
+    rows = bf(torch.randn(n, 3 * heads * dk + heads * dv, generator=g) * 2).to(DEV).to(dtype)
+    bias = bf(torch.randn(heads * dk, generator=g)).to(DEV).to(dtype)
+    qk = heads * dk
+    outs, states = [], []
+    for plan in ([[(0, 0, n)]], [[(0, p, 1)] for p in range(n)]):
+        state = torch.randn(1, heads, dk, dv, device=DEV)
+        run = lambda r, step: linear_scan(r[:, :qk], r[:, qk:2 * qk], r[:, 2 * qk:2 * qk + heads * dv], heads, dk, dv, step, state,  # noqa: E731
+                                          gate=r[:, 2 * qk + heads * dv:], gate_bias=bias, tau=3.0)
+        _, got = _walk(plan, {0: n}, dtype, lambda s, m: rows.cpu().float(), run)
+        outs.append(got[0])
+        states.append(state.clone())
+    assert torch.equal(outs[0], outs[1]) and torch.equal(states[0], states[1])
+
+
 @pytest.mark.parametrize("decay,far", [(1.0, 0), (0.998, 3), (0.998, 15), (0.998, 16), (0.99, 255)])
 def test_a_value_written_far_back_is_read_hundreds_of_tokens_later_through_many_portions(decay, far):
     """One key / value pair at position ``far`` is made large; a query that matches its key reads it 600 tokens later, scaled by
