@@ -720,7 +720,8 @@ int ll_moe_rows_gemm(const void* a, int64_t a_ld, int64_t a_div, const void* w, 
  * a = sigmoid(gate[t][h dk + i] + gate_bias[h dk + i])^inv_tau per key entry; kind 2: dt = softplus(dt[t][h] + dt_bias[h]),
  * a = exp(-exp(a_log[h]) dt), b = dt, skip [heads] or NULL.  o: fp32 [n, heads dv].  A run that starts at position 0 starts
  * from zeros.  decay_scratch (kind 1; fp32 [n, heads dk] for the step's n tokens, or NULL): the decays are evaluated once per
- * token and entry ahead of the scan instead of by every column workgroup (same values).
+ * token and entry ahead of the scan instead of by every column workgroup (same values).  longest_run: most tokens a sequence
+ * of the step brings (0: unknown); sizes the staging buffers only.
  * ll_gated_out_norm: o fp32 [n, width] -> RMS norm over `parts` equal consecutive parts, times w[(channel) mod w_len] (NULL:
  * none), times act(gate) (gate_kind 0 none, 1 silu, 2 sigmoid; gate_first: before the norm), times out_scale -> out rows of
  * stride out_ld.
@@ -736,7 +737,7 @@ int ll_linear_scan(const void* q, int64_t q_ld, const void* k, int64_t k_ld, con
                    const void* gate, int64_t gate_ld, const void* gate_bias, float inv_tau, const void* dt, int64_t dt_ld,
                    const void* dt_bias, const void* a_log, const void* skip, float* o, int64_t batch,
                    const int32_t* seq_start, const int32_t* seq_first_pos, const int32_t* seq_slot, float* state,
-                   float* decay_scratch, int64_t n, int dtype, void* stream);
+                   float* decay_scratch, int64_t n, int64_t longest_run, int dtype, void* stream);
 int ll_gated_out_norm(void* out, int64_t out_ld, const float* o, const void* gate, int64_t gate_ld, int gate_kind,
                       int gate_first, const void* w, int64_t w_len, float eps, float out_scale, int64_t n, int64_t width,
                       int64_t parts, int dtype, void* stream);

@@ -136,7 +136,7 @@ SIGNATURES = {
     "ll_moe_sort": [P, L, L, L, P, P, P, P, P],
     "ll_moe_rows_gemm": [P, L, L, P, L, L, L, I, P, P, L, P, P, P, L, L, L, F, I, P],
     "ll_linear_scan_supported": [L, L],
-    "ll_linear_scan": [P, L, P, L, P, L, L, L, L, L, I, I, F, P, P, L, P, F, P, L, P, P, P, P, L, P, P, P, P, P, L, I, P],
+    "ll_linear_scan": [P, L, P, L, P, L, L, L, L, L, I, I, F, P, P, L, P, F, P, L, P, P, P, P, L, P, P, P, P, P, L, L, I, P],
     "ll_gated_out_norm": [P, L, P, P, L, I, I, P, L, F, F, L, L, L, I, P],
     "ll_conv_act": [P, L, P, L, P, P, L, L, P, L, P, P, P, P, P, P, L, I, P],
     "ll_rownorm_rope_cache": [P, L, P, P, F, P, L, F, P, P, P, P, P, L, L, L, L, L, I, P],

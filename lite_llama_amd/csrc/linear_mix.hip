@@ -529,7 +529,7 @@ extern "C" int ll_linear_scan(const void* q, int64_t q_ld, const void* k, int64_
                               const void* gate, int64_t gate_ld, const void* gate_bias, float inv_tau, const void* dt, int64_t dt_ld,
                               const void* dt_bias, const void* a_log, const void* skip, float* o, int64_t batch,
                               const int32_t* seq_start, const int32_t* seq_first_pos, const int32_t* seq_slot, float* state,
-                              float* decay_scratch, int64_t n, int dtype, void* stream) {
+                              float* decay_scratch, int64_t n, int64_t longest_run, int dtype, void* stream) {
   if (dtype != LL_F16 && dtype != LL_BF16 && dtype != LL_F32) return LL_ERR_DTYPE;
   if (batch < 0 || heads < 1 || heads > 65535 || !ll_linear_scan_supported(dk, dv) || qk_rep < 1 || heads % qk_rep || kind < 0 ||
       kind > 2 || (dv + 15) / 16 > 65535)
@@ -547,7 +547,8 @@ extern "C" int ll_linear_scan(const void* q, int64_t q_ld, const void* k, int64_
   a.head_decay = head_decay; a.gate = gate; a.gate_ld = gate_ld; a.gate_bias = gate_bias; a.inv_tau = inv_tau;
   a.decay_pre = nullptr;
   a.dt = dt; a.dt_ld = dt_ld; a.dt_bias = dt_bias; a.a_log = a_log; a.skip = skip; a.o = o;
-  a.tb = dk <= 128 ? 16 : 8;
+  a.tb = dk <= 128 ? 16 : 8;   // tokens staged per pass; a step of short runs asks for less LDS and fits more workgroups per CU
+  if (longest_run > 0 && longest_run < a.tb) a.tb = (int)longest_run;
   a.seq_start = seq_start; a.seq_first_pos = seq_first_pos; a.seq_slot = seq_slot; a.state = state;
   const size_t lds = sizeof(float) * (size_t)(a.tb * (4 * dk + 16 + 16 + 256 + 2));
   const dim3 grid((unsigned)batch, (unsigned)heads, (unsigned)((dv + 15) / 16));

@@ -155,7 +155,7 @@ def linear_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, heads: int, d
         1 if act else 0, float(q_scale), L.ptr(head_decay), L.ptr(gate), gate.stride(0) if gate is not None else 0, L.ptr(gate_bias),
         1.0 / float(tau), L.ptr(dt), dt.stride(0) if dt is not None else 0, L.ptr(dt_bias), L.ptr(a_log), L.ptr(skip), o.data_ptr(),
         step.num_seqs, step.seq_start.data_ptr(), step.seq_first_pos.data_ptr(), step.seq_slot.data_ptr(), state.data_ptr(),
-        L.ptr(pre), n, L.dtype_code(st), L.stream_ptr()), "linear_scan")
+        L.ptr(pre), n, int(step.longest_run), L.dtype_code(st), L.stream_ptr()), "linear_scan")
     return o
 
 
